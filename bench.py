@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Decode-step benchmark of the DRAM Attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 128k] [--eager]
+
+A step is one `generate` call of one attention layer: page scoring, ordered
+top-k, LRU update, streaming of missed pages from pinned host DRAM, and decode
+attention over the resident pages + local window + new token.  Inputs of all
+steps are staged in HBM before the clock starts.  By default the step is
+captured once into a HIP graph (position and LRU step live on the device) and
+replayed; --eager issues the launches from Python every step.
+
+Prints ONE JSON line: the BASELINE metric plus `roofline` (dominant kernel,
+timed live with events on the launch stream) and `cpu_baseline` (the CPU oracle
+timed on this box's host cores on a bounded sample of the same workload).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="128k", choices=["cpu", "32k", "128k", "1m"])
+    ap.add_argument("--eager", action="store_true", help="no HIP graph: launch from Python each step")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--cpu-steps", type=int, default=8, help="steps of the CPU oracle to time (0 = skip)")
+    ap.add_argument("--profile-steps", type=int, default=16, help="extra steps timed per kernel with events")
+    return ap.parse_args()
+
+
+class Layer:
+    """One attention layer set up on the workload, plus the staged step inputs."""
+
+    def __init__(self, w, seed, total_steps, dev):
+        from dram_attention_amd import DRAMAttention
+        from dram_attention_amd.synthetic import DecodeInputs, make_prompt
+
+        self.w = w
+        prompt = make_prompt(w, seed)
+        self.prompt = prompt
+        self.m = DRAMAttention(max_output_length=total_steps, lru_hbm_cache_size=w.lru_tokens,
+                               local_cache_size=w.local_cache, page_size=w.page_size,
+                               top_k=w.top_k_tokens, n_kv_heads=w.n_kv_heads, head_dim=w.head_dim,
+                               device=dev, dtype=w.dtype)
+        self.m.init_cache(prompt.k.to(dev), prompt.v.to(dev))
+        inputs = DecodeInputs(w, prompt.q0, seed)
+        qs, ks, vs = zip(*(inputs.next() for _ in range(total_steps)))
+        self.host_inputs = (qs, ks, vs)
+        self.qs = torch.cat(qs).to(dev)   # (T, 1, Hq, D)
+        self.ks = torch.cat(ks).to(dev)
+        self.vs = torch.cat(vs).to(dev)
+        self.t_dev = torch.zeros(1, dtype=torch.int64, device=dev)          # step index
+        self.pos_dev = torch.full((1,), w.prompt_tokens, dtype=torch.int32, device=dev)
+        self.out = None
+
+    def step_from_device_state(self):
+        """One decode step driven entirely by device-resident counters."""
+        m = self.m
+        xq = self.qs.index_select(0, self.t_dev)
+        xk = self.ks.index_select(0, self.t_dev)
+        xv = self.vs.index_select(0, self.t_dev)
+        self.out = m(xq, xk, xv, start_pos=self.pos_dev, stage="generate")
+        self.t_dev += 1
+        self.pos_dev += 1
+        return self.out
+
+
+def algorithmic_bytes(w, local_rows):
+    e = torch.empty(0, dtype=w.dtype).element_size()
+    score = w.n_kv_heads * w.n_dram_pages * 2 * w.head_dim * e
+    attn = (w.n_hbm_pages * w.page_size + local_rows + 1) * w.n_kv_heads * 2 * w.head_dim * e
+    return score, attn
+
+
+def time_kernels(layer, steps):
+    """Per-entry-point GPU time, events recorded on the stream the kernels run on."""
+    from dram_attention_amd.dram_attention import decode_attention
+
+    m, lru = layer.m, layer.m.lru_cache
+    names = ("page_score", "topk_pages", "lru_update+pages_gather", "decode_attention")
+    acc = {n: 0.0 for n in names}
+    misses = 0
+    local_rows = []
+    for _ in range(steps):
+        t = int(layer.t_dev.item())
+        xq, xk, xv = layer.qs[t:t + 1], layer.ks[t:t + 1], layer.vs[t:t + 1]
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(5)]
+        sel = lru.top_k_selector
+        k = min(lru.top_k, lru.num_dram_pages)
+        ev[0].record()
+        scores = sel.scores(xq)
+        ev[1].record()
+        from dram_attention_amd.topk_selector import topk_pages
+        idx = lru._topk_idx
+        topk_pages(scores, layer.w.rep, k, idx, layer.w.rep * k, idx.shape[1], k)
+        ev[2].record()
+        pk, pv = lru.load_(idx)
+        ev[3].record()
+        c_len = int(layer.pos_dev.item()) - m.dram_kv_cache_size
+        out = decode_attention(xq[0, 0], pk, pv, m.cache_k[0], m.cache_v[0], c_len, xk[0, 0],
+                               xv[0, 0], workspace=m._workspace)
+        ev[4].record()
+        torch.cuda.synchronize()
+        for i, n in enumerate(names):
+            acc[n] += ev[i].elapsed_time(ev[i + 1])
+        misses += int(lru.last_miss_counts().sum().item())
+        local_rows.append(c_len)
+        layer.t_dev += 1
+        layer.pos_dev += 1
+    return ({n: v / steps * 1e3 for n, v in acc.items()},  # microseconds
+            misses / steps, sum(local_rows) / len(local_rows))
+
+
+def cpu_baseline(w, layer, steps):
+    """The CPU oracle (a restatement of the reference's torch/Triton path) on the
+    first `steps` decode steps of the same workload, all host cores."""
+    from oracle import dram_attention_oracle as O
+
+    o = O.DecodeOracle(steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                       w.n_kv_heads, w.head_dim, dtype=w.dtype)
+    o.init_cache(layer.prompt.k, layer.prompt.v)
+    qs, ks, vs = layer.host_inputs
+    t0 = time.perf_counter()
+    for t in range(steps):
+        o.generate(qs[t], ks[t], vs[t], w.prompt_tokens + t)
+    dt = time.perf_counter() - t0
+    return {"value": steps / dt, "unit": "decode steps/s per layer", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"first {steps} decode steps of workload {w.name}, torch-CPU oracle, "
+                      f"{dt / steps * 1e3:.1f} ms/step"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this hot path is a single-device decode step "
+              "(run with --gpus 1)", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the HIP kernels are the only implementation", file=sys.stderr)
+        return 2
+    from dram_attention_amd import _lib
+    from dram_attention_amd.synthetic import WORKLOADS
+
+    _lib.load()
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    w = WORKLOADS[args.workload]
+    total = args.warmup + args.steps + args.profile_steps + 4
+    layer = Layer(w, args.seed, total, dev)
+    torch.cuda.synchronize()
+
+    # -- warm-up (also resolves the pinned-host device address before any capture)
+    graph = None
+    if args.eager:
+        for _ in range(args.warmup):
+            layer.step_from_device_state()
+    else:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                layer.step_from_device_state()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            layer.step_from_device_state()
+        # the capture itself executed nothing; replay for the remaining warm-up steps
+        for _ in range(max(args.warmup - 2, 0)):
+            graph.replay()
+    torch.cuda.synchronize()
+
+    # -- timed region
+    t0 = time.perf_counter()
+    if graph is not None:
+        for _ in range(args.steps):
+            graph.replay()
+    else:
+        for _ in range(args.steps):
+            layer.step_from_device_state()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+
+    # -- per-kernel pass and traffic counters
+    kernel_us, miss_per_step, local_rows = time_kernels(layer, args.profile_steps)
+    score_b, attn_b = algorithmic_bytes(w, local_rows)
+    attn_us = kernel_us["decode_attention"]
+    achieved = attn_b / (attn_us * 1e-6) / 1e9
+    requests = w.n_kv_heads * w.rep * w.pages_per_q_head
+    page_bytes = w.page_size * 2 * w.head_dim * torch.empty(0, dtype=w.dtype).element_size()
+
+    result = {
+        "metric": "decode steps/sec per layer at 128K ctx; scorer+attn HBM GB/s vs peak",
+        "value": args.steps / dt,
+        "unit": "decode steps/s per layer",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[w.dtype],
+        "data": "synthetic",
+        "config": {
+            "workload": f"configs[{['cpu', '32k', '128k', '128k-x32', '1m'].index(w.name)}] {w.name}: "
+                        f"1 layer, {w.n_q_heads}q/{w.n_kv_heads}kv heads, D {w.head_dim}, "
+                        f"{w.dram_tokens}-token prefix in pinned host DRAM ({w.n_dram_pages} pages/head), "
+                        f"local {w.local_cache}, LRU {w.lru_tokens} tokens, top-k {w.top_k_tokens} tokens",
+            "launch": "eager" if args.eager else "hip-graph replay",
+            "seed": args.seed,
+        },
+        "roofline": {
+            "bound": "hbm", "kernel": "decode_attention (split + merge launches)",
+            "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "algorithmic_bytes": attn_b, "avg_us": attn_us,
+        },
+        "kernels_us": kernel_us,
+        "page_score_GBps": score_b / (kernel_us["page_score"] * 1e-6) / 1e9,
+        "lru": {"requests_per_step": requests, "distinct_misses_per_step": miss_per_step,
+                "h2d_bytes_per_step": miss_per_step * page_bytes},
+    }
+    if args.cpu_steps > 0:
+        result["cpu_baseline"] = cpu_baseline(w, layer, args.cpu_steps)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,22 @@
+"""DRAM Attention for AMD Instinct MI355X (gfx950): the reference package's
+Python surface on hand-written HIP kernels (libdramattn.so)."""
+
+__version__ = "0.1.0"
+
+from .dram_attention import DRAMAttention, decode_attention
+from .lru_cache import CacheOutput, DummyCache, LRUCache
+from .lru_kernel import load_lru_cache_
+from .max_ip_kernel import max_inner_product, max_ip_ref
+from .topk_selector import IPUpperboundTopKSelector
+
+__all__ = (
+    "CacheOutput",
+    "DRAMAttention",
+    "DummyCache",
+    "IPUpperboundTopKSelector",
+    "LRUCache",
+    "decode_attention",
+    "load_lru_cache_",
+    "max_inner_product",
+    "max_ip_ref",
+)

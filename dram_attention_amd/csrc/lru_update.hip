@@ -1,0 +1,323 @@
+// LRU lookup / touch / evict / slot-assign for one decode step, and the
+// grid-wide gather that fills the assigned slots from the DRAM page store.
+// Counterpart of dram_attention/lru_triton_kernel.py:6-194 of the reference.
+//
+// The reference walks the K requested pages of a head serially (one Triton
+// program per head) and needs a full stable argsort of the access times first.
+// When K <= N_hbm the walk is order-independent except for which victim each
+// distinct missed page receives, and that is fixed by ranks:
+//   the i-th distinct missed page (in visiting order) takes the slot with the
+//   i-th smallest (access_time, slot) after this step's hits were touched.
+// Proof sketch: touched slots carry the largest time, so they sort behind the
+// M <= K - T victims consumed; a victim's old page is resident and untouched,
+// hence not among the requests, so no later request observes the eviction.
+// So the kernel does: touch hits and mark first occurrences of missed pages
+// (atomicMax of a position marker in the page->slot map), rank those
+// occurrences with a block scan, select the M least-recent slots in order
+// (select_sorted), and rewrite both maps in parallel.
+// K > N_hbm (victims may wrap onto pages touched in the same step) keeps the
+// reference's literal serial walk on one lane per head.
+//
+// Bound: latency; algorithmic bytes are the metadata only.
+#include "select.hpp"
+
+namespace da {
+
+constexpr int kLruMaxK = 8192;  // distinct-miss list kept in LDS (parallel path)
+
+struct LruShared {
+  SelectShared sel;
+  int32_t miss_page[kLruMaxK];
+  uint32_t wave_count[kSelWaves];
+  uint32_t n_miss;
+};
+
+template <typename TimeT>
+__device__ __forceinline__ uint32_t time_order_key(TimeT v);
+template <>
+__device__ __forceinline__ uint32_t time_order_key<float>(float v) { return float_order_key(v); }
+template <>
+__device__ __forceinline__ uint32_t time_order_key<int32_t>(int32_t v) {
+  return (uint32_t)v ^ 0x80000000u;
+}
+
+// "largest key" = smallest access time, ties by lowest slot: the order of
+// torch.argsort(page_access_time, stable=True).
+template <typename TimeT>
+struct LeastRecentKey {
+  const TimeT *time;
+  __device__ __forceinline__ uint32_t operator()(int i) const {
+    return ~time_order_key<TimeT>(time[i]);
+  }
+};
+
+__device__ __forceinline__ void atomic_max_signed(int32_t *p, int32_t v) { atomicMax(p, v); }
+__device__ __forceinline__ void atomic_max_signed(int64_t *p, int64_t v) {
+  atomicMax((long long *)p, (long long)v);
+}
+
+template <typename IdxT, typename MapT, typename TimeT>
+__global__ void __launch_bounds__(kSelThreads)
+lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int K,
+                  int64_t n_dram_pages, int n_hbm, int32_t *step_ptr, int bump,
+                  TimeT *time_all, int64_t time_head_stride, MapT *d2h_all,
+                  int64_t d2h_head_stride, MapT *h2d_all, int64_t h2d_head_stride,
+                  uint8_t *hit_mask, int32_t *miss_page_out, int32_t *miss_slot_out,
+                  int32_t *miss_count, int32_t *ticket, int serial) {
+  __shared__ LruShared sm;
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = t >> 6;
+  const int h = blockIdx.x;
+  const IdxT *idx = idx_all + h * idx_head_stride;
+  TimeT *time = time_all + h * time_head_stride;
+  MapT *d2h = d2h_all + h * d2h_head_stride;
+  MapT *h2d = h2d_all + h * h2d_head_stride;
+  uint8_t *hit = hit_mask ? hit_mask + (int64_t)h * K : nullptr;
+  int32_t *mpage = miss_page_out + (int64_t)h * K;
+  int32_t *mslot = miss_slot_out + (int64_t)h * K;
+
+  const int32_t step = *step_ptr + (bump ? 1 : 0);
+  const TimeT now = (TimeT)step;
+
+  if (serial) {
+    // -- literal restatement of the reference's three launches ---------------
+    for (int k = t; k < K; k += kSelThreads) {
+      const int64_t p = (int64_t)idx[k];
+      if (p < 0 || p >= n_dram_pages) continue;
+      const int64_t s = (int64_t)d2h[p];
+      if (s >= 0) time[s] = now;
+    }
+    __syncthreads();
+    LeastRecentKey<TimeT> key{time};
+    select_sorted(key, n_hbm, n_hbm, sm.sel);  // full stable order of the slots
+    if (t == 0) {
+      int ep = 0, m = 0;
+      for (int k = 0; k < K; ++k) {
+        const int64_t p = (int64_t)idx[k];
+        if (p < 0 || p >= n_dram_pages) {
+          if (hit) hit[k] = 0;
+          continue;
+        }
+        const int64_t s = (int64_t)d2h[p];
+        if (s < 0) {
+          const int32_t v = (int32_t)sel_index(sm.sel.sel[ep]);
+          time[v] = now;
+          const int64_t old = (int64_t)h2d[v];
+          if (old >= 0) d2h[old] = (MapT)-1;
+          h2d[v] = (MapT)p;
+          d2h[p] = (MapT)v;
+          mpage[m] = (int32_t)p;
+          mslot[m] = v;
+          ++m;
+          ep = ep + 1 == n_hbm ? 0 : ep + 1;
+          if (hit) hit[k] = 0;
+        } else {
+          time[s] = now;
+          if (hit) hit[k] = 1;
+        }
+      }
+      sm.n_miss = (uint32_t)m;
+      miss_count[h] = m;
+    }
+    __syncthreads();
+    // an entry whose slot was handed out again later in the walk is dead
+    const int m = (int)sm.n_miss;
+    for (int i = t; i < m; i += kSelThreads)
+      if ((int64_t)h2d[mslot[i]] != (int64_t)mpage[i]) mslot[i] = -1;
+  } else {
+    // -- phase A: touch hits, mark the first occurrence of every missed page --
+    for (int k = t; k < K; k += kSelThreads) {
+      const int64_t p = (int64_t)idx[k];
+      if (p < 0 || p >= n_dram_pages) continue;
+      const int64_t s = (int64_t)d2h[p];
+      if (s >= 0)
+        time[s] = now;
+      else
+        atomic_max_signed(&d2h[p], (MapT)(-(int64_t)k - 2));  // smallest k wins
+    }
+    if (t == 0) sm.n_miss = 0;
+    __syncthreads();
+    // -- phase B: rank the first occurrences in visiting order ---------------
+    for (int base = 0; base < K; base += kSelThreads) {
+      const int k = base + t;
+      bool first = false;
+      int64_t p = -1;
+      if (k < K) {
+        p = (int64_t)idx[k];
+        if (p >= 0 && p < n_dram_pages) first = (int64_t)d2h[p] == -(int64_t)k - 2;
+        if (hit) hit[k] = (p >= 0 && p < n_dram_pages && !first) ? 1 : 0;
+      }
+      const uint64_t m_first = __ballot(first);
+      if (lane == 0) sm.wave_count[wave] = (uint32_t)__popcll(m_first);
+      __syncthreads();
+      uint32_t before = sm.n_miss, round = 0;
+#pragma unroll
+      for (int w = 0; w < kSelWaves; ++w) {
+        const uint32_t c = sm.wave_count[w];
+        if (w < wave) before += c;
+        round += c;
+      }
+      const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+      if (first) sm.miss_page[before + (uint32_t)__popcll(m_first & below)] = (int32_t)p;
+      __syncthreads();
+      if (t == 0) sm.n_miss += round;
+      __syncthreads();
+    }
+    const int m = (int)sm.n_miss;
+    // -- phase C: the m least recently used slots, in eviction order ---------
+    if (m > 0) {
+      LeastRecentKey<TimeT> key{time};
+      select_sorted(key, n_hbm, m, sm.sel);
+    }
+    // -- phase D: hand slot i to the i-th distinct missed page ---------------
+    for (int i = t; i < m; i += kSelThreads) {
+      const int32_t p = sm.miss_page[i];
+      const int32_t v = (int32_t)sel_index(sm.sel.sel[i]);
+      const int64_t old = (int64_t)h2d[v];
+      if (old >= 0) d2h[old] = (MapT)-1;
+      h2d[v] = (MapT)p;
+      d2h[p] = (MapT)v;
+      time[v] = now;
+      mpage[i] = p;
+      mslot[i] = v;
+    }
+    if (t == 0) miss_count[h] = m;
+  }
+
+  // The last head to finish publishes the bumped step (every head has read the
+  // old value by then) and re-arms the ticket for the next call.
+  if (bump && t == 0) {
+    __threadfence();
+    const int32_t done = atomicAdd(ticket, 1);
+    if (done == (int32_t)gridDim.x - 1) {
+      *step_ptr = step;
+      *ticket = 0;
+    }
+  }
+}
+
+// One 256-thread block per (entry, head), striding over the head's miss list.
+// Every lane moves 16 bytes at a time with all of a page's loads issued before
+// the first store, so a wave keeps several KiB of host-link reads in flight.
+__global__ void __launch_bounds__(256)
+pages_gather_kernel(const char *__restrict__ dram, int64_t dram_head_stride,
+                    int64_t dram_page_stride, char *__restrict__ hbm, int64_t hbm_head_stride,
+                    int64_t hbm_slot_stride, int64_t page_bytes,
+                    const int32_t *__restrict__ miss_page, const int32_t *__restrict__ miss_slot,
+                    const int32_t *__restrict__ miss_count, int K) {
+  const int h = blockIdx.y;
+  const int m = miss_count[h];
+  const int64_t vecs = page_bytes / 16;
+  for (int i = blockIdx.x; i < m; i += gridDim.x) {
+    const int32_t v = miss_slot[(int64_t)h * K + i];
+    if (v < 0) continue;
+    const int32_t p = miss_page[(int64_t)h * K + i];
+    const char *src = dram + h * dram_head_stride + p * dram_page_stride;
+    char *dst = hbm + h * hbm_head_stride + v * hbm_slot_stride;
+    for (int64_t j0 = threadIdx.x; j0 < vecs; j0 += 4 * 256) {
+      u32x4 r[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (j0 + u * 256 < vecs) r[u] = load16(src + (j0 + u * 256) * 16);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (j0 + u * 256 < vecs) store16(dst + (j0 + u * 256) * 16, r[u]);
+    }
+  }
+}
+
+template <typename IdxT, typename MapT>
+static void launch_lru_time(int time_type, dim3 grid, hipStream_t s, const void *idx,
+                            int64_t idx_hs, int K, int64_t P, int n_hbm, int32_t *step, int bump,
+                            void *time, int64_t time_hs, void *d2h, int64_t d2h_hs, void *h2d,
+                            int64_t h2d_hs, uint8_t *hit, int32_t *mp, int32_t *ms, int32_t *mc,
+                            int32_t *ticket, int serial) {
+  if (time_type == DA_TIME_F32)
+    hipLaunchKernelGGL((lru_update_kernel<IdxT, MapT, float>), grid, dim3(kSelThreads), 0, s,
+                       (const IdxT *)idx, idx_hs, K, P, n_hbm, step, bump, (float *)time, time_hs,
+                       (MapT *)d2h, d2h_hs, (MapT *)h2d, h2d_hs, hit, mp, ms, mc, ticket, serial);
+  else
+    hipLaunchKernelGGL((lru_update_kernel<IdxT, MapT, int32_t>), grid, dim3(kSelThreads), 0, s,
+                       (const IdxT *)idx, idx_hs, K, P, n_hbm, step, bump, (int32_t *)time,
+                       time_hs, (MapT *)d2h, d2h_hs, (MapT *)h2d, h2d_hs, hit, mp, ms, mc, ticket,
+                       serial);
+}
+
+}  // namespace da
+
+extern "C" size_t da_lru_update_workspace_bytes(int, int, int64_t, int) { return 256; }
+
+extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_itype,
+                             int n_kv_heads, int k, int64_t n_dram_pages, int n_hbm_pages,
+                             int32_t *step, int bump_step, void *access_time,
+                             int64_t time_head_stride, int time_type, void *d2h,
+                             int64_t d2h_head_stride, void *h2d, int64_t h2d_head_stride,
+                             int map_itype, uint8_t *hit_mask, int32_t *miss_page,
+                             int32_t *miss_slot, int32_t *miss_count, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+  using namespace da;
+  DA_REQUIRE(n_kv_heads >= 0 && k >= 0 && n_dram_pages >= 0 && n_hbm_pages >= 0,
+             "da_lru_update: bad geometry (heads %d k %d pages %lld slots %d)", n_kv_heads, k,
+             (long long)n_dram_pages, n_hbm_pages);
+  DA_REQUIRE(idx_itype == DA_I32 || idx_itype == DA_I64, "da_lru_update: bad idx type");
+  DA_REQUIRE(map_itype == DA_I32 || map_itype == DA_I64, "da_lru_update: bad map type");
+  DA_REQUIRE(time_type == DA_TIME_F32 || time_type == DA_TIME_I32,
+             "da_lru_update: bad access-time type");
+  if (n_kv_heads == 0) return DA_OK;
+  DA_REQUIRE(step && access_time && d2h && h2d && miss_page && miss_slot && miss_count,
+             "da_lru_update: null pointer");
+  DA_REQUIRE(k == 0 || idx, "da_lru_update: null index list");
+  DA_REQUIRE(workspace && workspace_bytes >= da_lru_update_workspace_bytes(0, 0, 0, 0),
+             "da_lru_update: workspace too small");
+  DA_REQUIRE(n_hbm_pages > 0 || k == 0, "da_lru_update: no HBM slots");
+  DA_REQUIRE(n_dram_pages <= 0x7fffffff, "da_lru_update: page ids must fit int32");
+  const int serial = (k > n_hbm_pages || k > kLruMaxK) ? 1 : 0;
+  if (serial && n_hbm_pages > kSelMaxK)
+    return fail(DA_ENOTSUP,
+                "da_lru_update: k %d > slots %d needs the serial walk, which orders at most %d "
+                "slots",
+                k, n_hbm_pages, kSelMaxK);
+  dim3 grid(n_kv_heads);
+  hipStream_t s = (hipStream_t)stream;
+  int32_t *ticket = (int32_t *)workspace;
+#define DA_LRU_ARGS                                                                          \
+  time_type, grid, s, idx, idx_head_stride, k, n_dram_pages, n_hbm_pages, step, bump_step,   \
+      access_time, time_head_stride, d2h, d2h_head_stride, h2d, h2d_head_stride, hit_mask,   \
+      miss_page, miss_slot, miss_count, ticket, serial
+  if (idx_itype == DA_I64 && map_itype == DA_I64)
+    launch_lru_time<int64_t, int64_t>(DA_LRU_ARGS);
+  else if (idx_itype == DA_I64)
+    launch_lru_time<int64_t, int32_t>(DA_LRU_ARGS);
+  else if (map_itype == DA_I64)
+    launch_lru_time<int32_t, int64_t>(DA_LRU_ARGS);
+  else
+    launch_lru_time<int32_t, int32_t>(DA_LRU_ARGS);
+#undef DA_LRU_ARGS
+  return launch_status("da_lru_update");
+}
+
+extern "C" int da_pages_gather(const void *dram, int64_t dram_head_stride_bytes,
+                               int64_t dram_page_stride_bytes, void *hbm,
+                               int64_t hbm_head_stride_bytes, int64_t hbm_slot_stride_bytes,
+                               int64_t page_bytes, const int32_t *miss_page,
+                               const int32_t *miss_slot, const int32_t *miss_count,
+                               int n_kv_heads, int k, void *stream) {
+  using namespace da;
+  DA_REQUIRE(n_kv_heads >= 0 && k >= 0 && page_bytes >= 0, "da_pages_gather: bad geometry");
+  if (n_kv_heads == 0 || k == 0 || page_bytes == 0) return DA_OK;
+  DA_REQUIRE(dram && hbm && miss_page && miss_slot && miss_count, "da_pages_gather: null pointer");
+  DA_REQUIRE(page_bytes % 16 == 0 && dram_head_stride_bytes % 16 == 0 &&
+                 dram_page_stride_bytes % 16 == 0 && hbm_head_stride_bytes % 16 == 0 &&
+                 hbm_slot_stride_bytes % 16 == 0 && (uintptr_t)dram % 16 == 0 &&
+                 (uintptr_t)hbm % 16 == 0,
+             "da_pages_gather: pages must be 16-byte aligned multiples of 16 bytes");
+  DA_REQUIRE(n_kv_heads <= 65535, "da_pages_gather: too many heads");
+  const int per_head = k < 128 ? k : 128;
+  dim3 grid(per_head, n_kv_heads);
+  hipLaunchKernelGGL(pages_gather_kernel, grid, dim3(256), 0, (hipStream_t)stream,
+                     (const char *)dram, dram_head_stride_bytes, dram_page_stride_bytes,
+                     (char *)hbm, hbm_head_stride_bytes, hbm_slot_stride_bytes, page_bytes,
+                     miss_page, miss_slot, miss_count, k);
+  return launch_status("da_pages_gather");
+}

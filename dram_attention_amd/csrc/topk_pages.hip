@@ -1,0 +1,68 @@
+// Ordered top-k page selection, one 1024-thread workgroup per score row.
+// Counterpart of torch.argsort(ip, descending=True)[..., :k] in
+// dram_attention/topk_selector.py:61 of the reference, with the tie order the
+// reference leaves open fixed to "lowest page index first" (a stable sort).
+//
+// Bound: latency (a row is a few tens of KiB and stays in L2); algorithmic
+// bytes = rows*P*4 read + rows*kp*8 written.
+#include "select.hpp"
+
+namespace da {
+
+struct ScoreKey {
+  const float *row;
+  __device__ __forceinline__ uint32_t operator()(int i) const { return float_order_key(row[i]); }
+};
+
+template <typename IdxT>
+__global__ void __launch_bounds__(kSelThreads)
+topk_pages_kernel(const float *__restrict__ scores, int64_t row_stride, int64_t head_stride,
+                  int rep, int n_pages, int kp, IdxT *__restrict__ out, int64_t out_seq_stride,
+                  int64_t out_head_stride, int64_t out_rep_stride) {
+  __shared__ SelectShared sm;
+  const int n = blockIdx.x;  // score row (query row)
+  const int h = blockIdx.y;
+  ScoreKey key{scores + n * row_stride + h * head_stride};
+  select_sorted(key, n_pages, kp, sm);
+  IdxT *dst = out + (n / rep) * out_seq_stride + h * out_head_stride + (n % rep) * out_rep_stride;
+  for (int j = threadIdx.x; j < kp; j += kSelThreads) dst[j] = (IdxT)sel_index(sm.sel[j]);
+}
+
+}  // namespace da
+
+extern "C" size_t da_topk_pages_workspace_bytes(int, int, int64_t, int) { return 0; }
+
+extern "C" int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
+                             int n_rows, int rep, int n_heads, int64_t n_pages, int kp, void *out,
+                             int64_t out_seq_stride, int64_t out_head_stride,
+                             int64_t out_rep_stride, int out_itype, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+  using namespace da;
+  (void)workspace;
+  (void)workspace_bytes;
+  DA_REQUIRE(n_rows >= 0 && n_heads >= 0 && n_pages >= 0 && kp >= 0 && rep >= 1,
+             "da_topk_pages: bad geometry (rows %d heads %d pages %lld kp %d rep %d)", n_rows,
+             n_heads, (long long)n_pages, kp, rep);
+  DA_REQUIRE(kp <= n_pages, "da_topk_pages: kp %d exceeds the %lld pages of a row", kp,
+             (long long)n_pages);
+  DA_REQUIRE(out_itype == DA_I32 || out_itype == DA_I64, "da_topk_pages: bad index type %d",
+             out_itype);
+  if (n_rows == 0 || n_heads == 0 || kp == 0) return DA_OK;
+  DA_REQUIRE(scores && out, "da_topk_pages: null pointer");
+  if (kp > kSelMaxK)
+    return fail(DA_ENOTSUP, "da_topk_pages: kp %d above the %d survivors sorted in LDS", kp,
+                kSelMaxK);
+  if (n_pages > 0x7fffffff || n_heads > 65535)
+    return fail(DA_ENOTSUP, "da_topk_pages: row length or head count out of range");
+  dim3 grid(n_rows, n_heads);
+  hipStream_t s = (hipStream_t)stream;
+  if (out_itype == DA_I64)
+    hipLaunchKernelGGL(topk_pages_kernel<int64_t>, grid, dim3(kSelThreads), 0, s, scores,
+                       row_stride, head_stride, rep, (int)n_pages, kp, (int64_t *)out,
+                       out_seq_stride, out_head_stride, out_rep_stride);
+  else
+    hipLaunchKernelGGL(topk_pages_kernel<int32_t>, grid, dim3(kSelThreads), 0, s, scores,
+                       row_stride, head_stride, rep, (int)n_pages, kp, (int32_t *)out,
+                       out_seq_stride, out_head_stride, out_rep_stride);
+  return launch_status("da_topk_pages");
+}

@@ -1,0 +1,219 @@
+"""DRAM Attention: long prefix in pinned host DRAM, hot pages in an HBM LRU,
+recent tokens in a local HBM window; decode attends over (resident pages ++
+local window ++ new token) in one split-K pass.
+
+Mirrors dram_attention/dram_attention.py of the reference (DRAMAttention
+:7-238): constructor, buffers, ``init_cache`` and ``forward(xq, xk, xv, *,
+start_pos, stage)`` keep their meaning and error behaviour.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+from . import _lib
+from .lru_cache import DummyCache, LRUCache
+
+
+def decode_attention(
+    xq: torch.Tensor,
+    prefix_k: torch.Tensor,
+    prefix_v: torch.Tensor,
+    cache_k: torch.Tensor,
+    cache_v: torch.Tensor,
+    cache_len,
+    new_k: torch.Tensor | None,
+    new_v: torch.Tensor | None,
+    *,
+    workspace: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
+    lse: torch.Tensor | None = None,
+    scale: float | None = None,
+) -> torch.Tensor:
+    """One query token against [prefix ++ cache rows 0..cache_len ++ new token].
+
+    xq (Hq, D); prefix_k/v (Hkv, T, D) views with a dense last axis (T may be 0);
+    cache_k/v (capacity, Hkv, D); cache_len an int or a one-element int32 GPU
+    tensor; new_k/new_v (Hkv, D) are appended at row cache_len (or None).
+    Returns (Hq, D) in xq.dtype; fills ``lse`` (Hq, fp32) when given.
+    """
+    Hq, D = xq.shape
+    Hkv = cache_k.shape[1]
+    _lib.require_gpu(xq, "xq")
+    lib = _lib.load()
+    dt = _lib.dtype_code(xq.dtype)
+    p_len = prefix_k.shape[1] if prefix_k is not None else 0
+    capacity = cache_k.shape[0]
+    if out is None:
+        out = torch.empty(Hq, D, dtype=xq.dtype, device=xq.device)
+    need = lib.da_decode_attention_workspace_bytes(Hq, Hkv, D, dt, p_len, capacity)
+    if need == 0:
+        raise RuntimeError(f"decode attention does not cover head_dim={D} dtype={xq.dtype}")
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty((need + 3) // 4, dtype=torch.float32, device=xq.device)
+    if isinstance(cache_len, torch.Tensor):
+        _lib.require_gpu(cache_len, "cache_len")
+        if cache_len.dtype != torch.int32:
+            raise TypeError("a device-side cache length must be int32")
+        len_host, len_dev = 0, cache_len.data_ptr()
+    else:
+        len_host, len_dev = int(cache_len), None
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    for t in (xq, prefix_k, prefix_v, cache_k, cache_v, new_k, new_v):
+        if t is not None and t.numel() and t.stride(-1) != 1:
+            raise ValueError("head_dim must be the dense axis of every operand")
+    _lib.check(
+        lib.da_decode_attention(
+            xq.data_ptr(), xq.stride(0), Hq, Hkv, D, dt,
+            prefix_k.data_ptr() if p_len else None, prefix_v.data_ptr() if p_len else None,
+            prefix_k.stride(1) if p_len else 0, prefix_k.stride(0) if p_len else 0, p_len,
+            cache_k.data_ptr(), cache_v.data_ptr(), cache_k.stride(0), cache_k.stride(1),
+            capacity, len_host, len_dev,
+            new_k.data_ptr() if new_k is not None else None,
+            new_v.data_ptr() if new_v is not None else None,
+            new_k.stride(0) if new_k is not None else 0,
+            scale, out.data_ptr(), out.stride(0),
+            lse.data_ptr() if lse is not None else None,
+            workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+            _lib.stream_ptr(xq.device),
+        ),
+        "da_decode_attention",
+    )
+    return out
+
+
+def causal_prefill_attention(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor) -> torch.Tensor:
+    """Dense causal attention over the prompt, (1,S,Hq,D) -> (1,S,Hq,D).  Not on
+    the decode path; torch's fused SDPA stands in for flash_attn_func
+    (reference dram_attention.py:136).  If no fused kernel takes the shape,
+    queries go in blocks so that no S x S score matrix is ever materialised."""
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+
+    bsz, S, Hq, D = xq.shape
+    Hkv = xk.shape[2]
+    q = xq.transpose(1, 2)
+    k = xk.transpose(1, 2)
+    v = xv.transpose(1, 2)
+    gqa = Hq != Hkv
+    if xq.is_cuda:
+        try:
+            with sdpa_kernel([SDPBackend.FLASH_ATTENTION, SDPBackend.EFFICIENT_ATTENTION]):
+                o = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=gqa)
+            return o.transpose(1, 2).contiguous()
+        except RuntimeError:
+            pass
+    out = torch.empty_like(xq)
+    block = 1024
+    for s0 in range(0, S, block):
+        s1 = min(S, s0 + block)
+        # rows s0..s1 see keys 0..s1; row i of the block may look at key j <= s0 + i
+        mask = torch.ones(s1 - s0, s1, dtype=torch.bool, device=xq.device).tril_(diagonal=s0)
+        o = F.scaled_dot_product_attention(q[:, :, s0:s1], k[:, :, :s1], v[:, :, :s1],
+                                           attn_mask=mask, enable_gqa=gqa)
+        out[:, s0:s1] = o.transpose(1, 2)
+    return out
+
+
+class DRAMAttention(torch.nn.Module):
+    """Drop-in for the reference module of the same name.
+
+    Two caches: ``cache_k/cache_v`` hold the local window (last
+    ``local_cache_size`` prompt tokens, rounded to pages, plus everything
+    generated); the rest of the prompt is paged, in host DRAM behind an
+    ``LRUCache`` (or entirely in HBM behind a ``DummyCache`` when it fits
+    into ``lru_hbm_cache_size``).
+    """
+
+    def __init__(
+        self,
+        max_output_length: int,
+        lru_hbm_cache_size: int,
+        local_cache_size: int,
+        page_size: int,
+        top_k: int,
+        n_kv_heads: int,
+        head_dim: int,
+        device: str = "cuda",
+        dtype: torch.dtype = torch.bfloat16,
+    ):
+        super().__init__()
+        self.max_output_length = max_output_length
+        self.page_size = page_size
+        self.dram_kv_cache_size = None  # set by init_cache
+        self.lru_hbm_cache_size = lru_hbm_cache_size
+        self.local_cache_size = local_cache_size
+        self.top_k = top_k
+        self.n_kv_heads = n_kv_heads
+        self.head_dim = head_dim
+        self.num_page = self.lru_hbm_cache_size // self.page_size
+        self.device = device
+        cache_shape = (1, local_cache_size + max_output_length, n_kv_heads, head_dim)
+        self.register_buffer("cache_k", torch.zeros(cache_shape, device=device, dtype=dtype))
+        self.register_buffer("cache_v", torch.zeros(cache_shape, device=device, dtype=dtype))
+        self._workspace = None
+
+    def init_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor):
+        """Split the prompt's (1,S,Hkv,D) keys/values into the paged prefix and the
+        local window, and build the page cache."""
+        bsz, seqlen, H, D = k_cache.shape
+        assert bsz == 1, "Only support batch size 1"
+        paged = (seqlen - self.local_cache_size + self.page_size) // self.page_size
+        self.dram_kv_cache_size = paged * self.page_size
+        tail = seqlen - self.dram_kv_cache_size
+        self.cache_k[:, :tail].copy_(k_cache[:, self.dram_kv_cache_size:], non_blocking=True)
+        self.cache_v[:, :tail].copy_(v_cache[:, self.dram_kv_cache_size:], non_blocking=True)
+        prefix_k = k_cache[0, : self.dram_kv_cache_size].transpose(0, 1)
+        prefix_v = v_cache[0, : self.dram_kv_cache_size].transpose(0, 1)
+        if self.dram_kv_cache_size > self.lru_hbm_cache_size:
+            self.lru_cache = LRUCache(
+                k_cache=prefix_k,
+                v_cache=prefix_v,
+                page_size=self.page_size,
+                top_k=self.top_k // self.page_size,
+                lru_hbm_cache_size=self.lru_hbm_cache_size,
+                device=self.device,
+            )
+        else:
+            self.lru_cache = DummyCache(k_cache=prefix_k, v_cache=prefix_v, device=self.device)
+        self._workspace = None
+
+    def forward(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, *, start_pos,
+                stage: str):
+        bsz, seqlen, H, D = xq.shape
+        assert bsz == 1, "Only support batch size 1"
+        if stage == "prefill":
+            output = causal_prefill_attention(xq, xk, xv)
+            self.init_cache(xk, xv)
+            return output
+        elif stage == "generate":
+            return self._generate(xq, xk, xv, start_pos)
+        else:
+            raise RuntimeError(f"Unsupported stage: {stage}")
+
+    def _generate(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, start_pos):
+        """One decode step: page in what the query needs, then one attention pass
+        over resident pages, local window and the new token (appended in place)."""
+        bsz, seqlen, Hq, D = xq.shape
+        if seqlen != 1:
+            raise RuntimeError("generate handles one token per call")
+        prefix_k, prefix_v = self.lru_cache.get_kv_cache_(xq)
+        if isinstance(start_pos, torch.Tensor):
+            cache_len = (start_pos - self.dram_kv_cache_size).to(torch.int32).reshape(1)
+        else:
+            cache_len = int(start_pos) - self.dram_kv_cache_size
+        if self._workspace is None:
+            lib = _lib.load()
+            need = lib.da_decode_attention_workspace_bytes(
+                Hq, self.n_kv_heads, D, _lib.dtype_code(xq.dtype), prefix_k.shape[1],
+                self.cache_k.shape[1])
+            self._workspace = torch.empty((need + 3) // 4, dtype=torch.float32, device=xq.device)
+        out = torch.empty(1, 1, Hq, D, dtype=xq.dtype, device=xq.device)
+        decode_attention(
+            xq[0, 0], prefix_k, prefix_v, self.cache_k[0], self.cache_v[0], cache_len,
+            xk[0, 0], xv[0, 0], workspace=self._workspace, out=out[0, 0],
+        )
+        return out

@@ -1,0 +1,129 @@
+"""LRU lookup / evict / slot-assign and page streaming on HIP kernels.
+
+Mirrors dram_attention/lru_triton_kernel.py of the reference:
+``load_lru_cache_`` (:140-194) keeps its signature and in-place semantics.
+"""
+
+from __future__ import annotations
+
+from typing import NamedTuple, Optional
+
+import torch
+
+from . import _lib
+
+
+class LruScratch(NamedTuple):
+    """Per-cache device buffers the two kernels exchange (allocated once)."""
+
+    miss_page: torch.Tensor   # (H, K) int32: i-th distinct missed page of a head
+    miss_slot: torch.Tensor   # (H, K) int32: the slot it was given
+    miss_count: torch.Tensor  # (H,) int32
+    hit_mask: torch.Tensor    # (H, K) uint8: 1 = resident when visited
+    workspace: torch.Tensor   # zeroed once; holds the step-bump ticket
+
+    @staticmethod
+    def allocate(num_heads: int, k: int, device) -> "LruScratch":
+        lib = _lib.load()
+        ws = lib.da_lru_update_workspace_bytes(num_heads, k, 0, 0)
+        return LruScratch(
+            miss_page=torch.empty(num_heads, max(k, 1), dtype=torch.int32, device=device),
+            miss_slot=torch.empty(num_heads, max(k, 1), dtype=torch.int32, device=device),
+            miss_count=torch.zeros(num_heads, dtype=torch.int32, device=device),
+            hit_mask=torch.empty(num_heads, max(k, 1), dtype=torch.uint8, device=device),
+            workspace=torch.zeros(ws, dtype=torch.uint8, device=device),
+        )
+
+
+def lru_update_and_gather(
+    dram_kv_cache: torch.Tensor,
+    page_access_time: torch.Tensor,
+    dram_page_to_hbm_page_mapping: torch.Tensor,
+    hbm_page_to_dram_page_mapping: torch.Tensor,
+    topk_dram_page_index: torch.Tensor,
+    current_step: torch.Tensor,
+    hbm_kv_cache: torch.Tensor,
+    scratch: LruScratch,
+    bump_step: bool,
+    dram_device_ptr: Optional[int] = None,
+) -> None:
+    """Two launches on the current stream: metadata update, then page gather."""
+    num_heads, num_dram_pages, page_dim = dram_kv_cache.shape
+    _, k = topk_dram_page_index.shape
+    assert (
+        dram_kv_cache.shape[0] == hbm_kv_cache.shape[0]
+        and dram_kv_cache.shape[2] == hbm_kv_cache.shape[2]
+    )
+    num_hbm_pages = hbm_kv_cache.shape[1]
+    if scratch.miss_page.shape != (num_heads, max(k, 1)):
+        raise ValueError("scratch was allocated for another (heads, k)")
+    for name, t in (("page_access_time", page_access_time),
+                    ("dram_page_to_hbm_page_mapping", dram_page_to_hbm_page_mapping),
+                    ("hbm_page_to_dram_page_mapping", hbm_page_to_dram_page_mapping),
+                    ("topk_dram_page_index", topk_dram_page_index),
+                    ("current_step", current_step), ("hbm_kv_cache", hbm_kv_cache)):
+        _lib.require_gpu(t, name)
+        if t.dim() > 1 and t.shape[-1] > 1 and t.stride(-1) != 1:
+            raise ValueError(f"{name} must be dense along its last axis")
+    if dram_page_to_hbm_page_mapping.dtype != hbm_page_to_dram_page_mapping.dtype:
+        raise TypeError("the two page mappings must share one integer type")
+    if current_step.dtype != torch.int32:
+        raise TypeError("current_step must be int32")
+    if dram_kv_cache.dtype != hbm_kv_cache.dtype:
+        raise TypeError("DRAM and HBM page stores must share one element type")
+    if dram_kv_cache.stride(2) != 1 or hbm_kv_cache.stride(2) != 1:
+        raise ValueError("pages must be dense")
+    dev = hbm_kv_cache.device
+    lib = _lib.load()
+    stream = _lib.stream_ptr(dev)
+    _lib.check(
+        lib.da_lru_update(
+            topk_dram_page_index.data_ptr(), topk_dram_page_index.stride(0),
+            _lib.itype_code(topk_dram_page_index.dtype), num_heads, k, num_dram_pages,
+            num_hbm_pages, current_step.data_ptr(), int(bump_step),
+            page_access_time.data_ptr(), page_access_time.stride(0),
+            _lib.time_code(page_access_time.dtype),
+            dram_page_to_hbm_page_mapping.data_ptr(), dram_page_to_hbm_page_mapping.stride(0),
+            hbm_page_to_dram_page_mapping.data_ptr(), hbm_page_to_dram_page_mapping.stride(0),
+            _lib.itype_code(dram_page_to_hbm_page_mapping.dtype),
+            scratch.hit_mask.data_ptr(), scratch.miss_page.data_ptr(),
+            scratch.miss_slot.data_ptr(), scratch.miss_count.data_ptr(),
+            scratch.workspace.data_ptr(), scratch.workspace.numel(), stream,
+        ),
+        "da_lru_update",
+    )
+    if dram_device_ptr is None:
+        dram_device_ptr = _lib.device_visible_ptr(dram_kv_cache)
+    esz = dram_kv_cache.element_size()
+    _lib.check(
+        lib.da_pages_gather(
+            dram_device_ptr, dram_kv_cache.stride(0) * esz, dram_kv_cache.stride(1) * esz,
+            hbm_kv_cache.data_ptr(), hbm_kv_cache.stride(0) * esz, hbm_kv_cache.stride(1) * esz,
+            page_dim * esz, scratch.miss_page.data_ptr(), scratch.miss_slot.data_ptr(),
+            scratch.miss_count.data_ptr(), num_heads, k, stream,
+        ),
+        "da_pages_gather",
+    )
+
+
+def load_lru_cache_(
+    dram_kv_cache: torch.Tensor,
+    page_access_time: torch.Tensor,
+    dram_page_to_hbm_page_mapping: torch.Tensor,
+    hbm_page_to_dram_page_mapping: torch.Tensor,
+    topk_dram_page_index: torch.Tensor,
+    *,
+    current_step: torch.Tensor,
+    hbm_kv_cache: torch.Tensor,
+):
+    """Touch / evict / assign / copy for one step, in place, as the reference's
+    function of the same name; metadata may be int32 or int64, access times
+    float32 or int32, the page store a GPU tensor or pinned host memory."""
+    num_heads = dram_kv_cache.shape[0]
+    k = topk_dram_page_index.shape[1]
+    scratch = LruScratch.allocate(num_heads, k, hbm_kv_cache.device)
+    lru_update_and_gather(
+        dram_kv_cache, page_access_time, dram_page_to_hbm_page_mapping,
+        hbm_page_to_dram_page_mapping, topk_dram_page_index, current_step, hbm_kv_cache,
+        scratch, bump_step=False,
+    )

@@ -1,0 +1,113 @@
+"""Quest page selector on HIP kernels (page summaries, scores, ordered top-k).
+
+Mirrors dram_attention/topk_selector.py of the reference
+(IPUpperboundTopKSelector: __init__ :16-35, top_k :37-61).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .max_ip_kernel import page_scores
+
+
+def page_min_max(k_cache: torch.Tensor, num_pages: int) -> torch.Tensor:
+    """(H, S, D) keys -> (H, num_pages, 2, D) per-page channel min ([..,0,:]) and max."""
+    num_heads, length, head_dim = k_cache.shape
+    assert length % num_pages == 0, "Cache size must be divisible by num_pages."
+    _lib.require_gpu(k_cache, "k_cache")
+    if k_cache.stride(-1) != 1:
+        k_cache = k_cache.contiguous()
+    page = length // num_pages
+    out = torch.empty(num_heads, num_pages, 2, head_dim, dtype=k_cache.dtype,
+                      device=k_cache.device)
+    lib = _lib.load()
+    _lib.check(
+        lib.da_page_minmax(
+            k_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1), num_heads, num_pages,
+            page, head_dim, _lib.dtype_code(k_cache.dtype), out.data_ptr(),
+            _lib.stream_ptr(k_cache.device),
+        ),
+        "da_page_minmax",
+    )
+    return out
+
+
+def topk_pages(scores: torch.Tensor, rep: int, k: int, out: torch.Tensor,
+               seq_stride: int, head_stride: int, rep_stride: int) -> torch.Tensor:
+    """Ordered top-k of every row of fp32 ``scores`` (n_rows, H, L); row n of head h
+    lands at (n // rep)*seq_stride + h*head_stride + (n % rep)*rep_stride in ``out``."""
+    n_rows, H, L = scores.shape
+    assert scores.dtype == torch.float32 and (L <= 1 or scores.stride(-1) == 1)
+    lib = _lib.load()
+    _lib.check(
+        lib.da_topk_pages(
+            scores.data_ptr(), scores.stride(0), scores.stride(1), n_rows, rep, H, L, k,
+            out.data_ptr(), seq_stride, head_stride, rep_stride, _lib.itype_code(out.dtype),
+            None, 0, _lib.stream_ptr(scores.device),
+        ),
+        "da_topk_pages",
+    )
+    return out
+
+
+class IPUpperboundTopKSelector:
+    """Inner-product upper-bound top-k page selector (Quest).
+
+    Ranking contract: pages are ordered by descending score and, among equal
+    scores, by ascending page index (the reference's argsort leaves ties open).
+    Scores of 16-bit inputs are rounded to the input type before ranking, as the
+    reference's kernel output is.
+    """
+
+    def __init__(self, k_cache: torch.Tensor, num_pages: int, device="cuda"):
+        num_heads, dram_kv_cache_size, head_dim = k_cache.shape
+        self.num_kv_heads = num_heads
+        assert dram_kv_cache_size % num_pages == 0, "Cache size must be divisible by num_pages."
+        self.device = torch.device(device)
+        # the summaries are built on the GPU: host-resident keys are moved first
+        self.chunk_min_max = page_min_max(k_cache.to(device=device), num_pages)
+        self._scores = None
+
+    def scores(self, q: torch.Tensor) -> torch.Tensor:
+        """fp32 scores (seq_len*rep, num_kv_heads, num_pages); row s*rep + r is query
+        head h*rep + r of token s."""
+        bsz, seq_len, num_q_heads, head_dim = q.shape
+        assert bsz == 1, f"Only batch size 1 is supported, but got batch size {bsz}"
+        assert num_q_heads % self.num_kv_heads == 0
+        rep = num_q_heads // self.num_kv_heads
+        H, L = self.num_kv_heads, self.chunk_min_max.shape[1]
+        if q.stride(-1) != 1:
+            q = q.contiguous()
+        n_rows = seq_len * rep
+        if self._scores is None or self._scores.shape[0] != n_rows:
+            self._scores = torch.empty(n_rows, H, L, dtype=torch.float32, device=q.device)
+        if seq_len == 1:
+            # (rep, H, D) view of the single token's heads: strides (D, rep*D, 1)
+            qv = q[0, 0].view(H, rep, head_dim).transpose(0, 1)
+        else:
+            qv = q[0].view(seq_len, H, rep, head_dim).transpose(1, 2).reshape(n_rows, H, head_dim)
+        return page_scores(qv, self.chunk_min_max, self._scores, round_to_input=True)
+
+    def top_k(self, q: torch.Tensor, k: int) -> torch.Tensor:
+        """Indices of the top k pages, (seq_len, num_kv_heads, rep, k) int64, best first."""
+        bsz, seq_len, num_q_heads, _ = q.shape
+        scores = self.scores(q)
+        rep = num_q_heads // self.num_kv_heads
+        H, L = self.num_kv_heads, scores.shape[-1]
+        k = min(k, L)
+        out = torch.empty(seq_len, H, rep, k, dtype=torch.int64, device=q.device)
+        return topk_pages(scores, rep, k, out, H * rep * k, rep * k, k)
+
+    def top_k_for_lru(self, q: torch.Tensor, k: int, out: torch.Tensor | None = None):
+        """The same selection laid out as the LRU consumes it, (num_kv_heads,
+        seq_len*rep*k): what swapaxes(0,1).contiguous().view(H,-1) of top_k gives."""
+        bsz, seq_len, num_q_heads, _ = q.shape
+        scores = self.scores(q)
+        rep = num_q_heads // self.num_kv_heads
+        H, L = self.num_kv_heads, scores.shape[-1]
+        k = min(k, L)
+        if out is None:
+            out = torch.empty(H, seq_len * rep * k, dtype=torch.int64, device=q.device)
+        return topk_pages(scores, rep, k, out, rep * k, seq_len * rep * k, k)

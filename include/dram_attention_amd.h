@@ -1,0 +1,197 @@
+/*
+ * C ABI of libdramattn.so — hand-written gfx950 (MI355X) kernels for the
+ * generate-stage hot path of DRAM Attention.
+ *
+ * The reference (a pure-Python package) has no FFI of its own; every entry
+ * point below replaces a Triton kernel, a torch op or a flash-attn call on the
+ * reference's decode path and cites it.  Conventions shared by all calls:
+ *
+ *   - plain C types only; every pointer is BORROWED device-accessible memory
+ *     (HBM, or pinned host memory mapped into the device address space);
+ *   - strides are in ELEMENTS of the tensor's dtype unless the name ends in
+ *     `_bytes`; the innermost (head_dim) axis is always contiguous;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *     default stream) and the call returns without synchronising;
+ *   - nothing is allocated or freed; scratch memory comes in through
+ *     `workspace` arguments whose size the matching *_workspace_bytes() gives;
+ *   - the return value is DA_OK (0), a negative DA_E* code for a rejected
+ *     argument (nothing was launched), or a positive hipError_t from the
+ *     launch; da_last_error_string() describes the last failure of the
+ *     calling thread.
+ */
+#ifndef DRAM_ATTENTION_AMD_H
+#define DRAM_ATTENTION_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DA_OK 0
+#define DA_EINVAL (-1)  /* malformed argument (null pointer, bad size, bad dtype) */
+#define DA_ENOTSUP (-2) /* well-formed but outside what the kernels cover */
+
+/* element types of K/V/q tensors */
+#define DA_F32 0
+#define DA_F16 1
+#define DA_BF16 2
+/* integer types of index / mapping tensors, and of page_access_time */
+#define DA_I32 0
+#define DA_I64 1
+#define DA_TIME_F32 0
+#define DA_TIME_I32 1
+
+/* Library version: major*10000 + minor*100 + patch. */
+int da_version(void);
+
+/* Text for the last non-zero return value on this thread ("" if none). */
+const char *da_last_error_string(void);
+
+/*
+ * Device-visible address of a pinned (hipHostMalloc'd) host buffer, so that
+ * kernels can read pages straight out of host DRAM.  Replaces the implicit UVA
+ * dereference of the pinned `dram_kv_cache` tensor inside
+ * dram_attention/lru_triton_kernel.py:81-89.
+ */
+int da_host_device_pointer(const void *host_ptr, void **device_ptr);
+
+/*
+ * Subsystem 1 — per-page, per-channel min and max of the keys.
+ * Replaces torch.aminmax + torch.stack in
+ * dram_attention/topk_selector.py:31-34.
+ *   k        : (Hkv, P*page, D) keys, element strides (k_head_stride, k_tok_stride, 1)
+ *   out      : (Hkv, P, 2, D) contiguous, same dtype; [...,0,:] = min, [...,1,:] = max
+ * NaNs propagate as in torch.aminmax.
+ */
+int da_page_minmax(const void *k, int64_t k_head_stride, int64_t k_tok_stride,
+                   int n_kv_heads, int64_t n_pages, int page_size, int head_dim,
+                   int dtype, void *out, void *stream);
+
+/*
+ * Subsystem 2 — Quest upper-bound page score
+ *     score[n,h,l] = sum_d max(q[n,h,d]*mm[h,l,0,d], q[n,h,d]*mm[h,l,1,d]).
+ * Replaces _max_inner_product_kernel / max_inner_product in
+ * dram_attention/max_ip_triton_kernel.py:20-124 (formula: max_ip_ref, :127-133).
+ *   q      : (n_rows, H, D), element strides (q_row_stride, q_head_stride, 1)
+ *   minmax : (H, L, 2, D), element strides (mm_head_stride, mm_page_stride, mm_r_stride, 1)
+ *   out    : (n_rows, H, L) with element strides (out_row_stride, out_head_stride, 1);
+ *            out_dtype is DA_F32 or equal to `dtype`.
+ * Arithmetic follows the reference kernel: for 16-bit inputs each product is
+ * rounded to the input type, the maximum and the sum over D are fp32; when
+ * `round_to_input` is non-zero the fp32 sum is rounded to the input type
+ * before it is stored (the value the reference ranks on, :99), also when
+ * out_dtype is DA_F32.
+ */
+int da_page_score(const void *q, int64_t q_row_stride, int64_t q_head_stride,
+                  const void *minmax, int64_t mm_head_stride, int64_t mm_page_stride,
+                  int64_t mm_r_stride, int n_rows, int n_heads, int64_t n_pages,
+                  int head_dim, int dtype, void *out, int64_t out_row_stride,
+                  int64_t out_head_stride, int out_dtype, int round_to_input,
+                  void *stream);
+
+/*
+ * Subsystem 3 — ordered top-k page selection per score row.
+ * Replaces torch.argsort(ip, descending=True)[..., :k] in
+ * dram_attention/topk_selector.py:61 and the layout shuffle in
+ * dram_attention/lru_cache.py:263-264.
+ *   scores : fp32, row (n, h) starts at n*row_stride + h*head_stride, n_pages long
+ *   out    : the kp page indices of row (n, h), best first, written at
+ *            (n / rep)*out_seq_stride + h*out_head_stride + (n % rep)*out_rep_stride
+ * Order: descending score; equal scores by ascending page index (a stable
+ * descending sort).  -0.0 equals +0.0; NaN ranks above +inf (torch's order).
+ * workspace: da_topk_pages_workspace_bytes(...) bytes, no initial state needed.
+ */
+size_t da_topk_pages_workspace_bytes(int n_rows, int n_heads, int64_t n_pages, int kp);
+int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
+                  int n_rows, int rep, int n_heads, int64_t n_pages, int kp,
+                  void *out, int64_t out_seq_stride, int64_t out_head_stride,
+                  int64_t out_rep_stride, int out_itype, void *workspace,
+                  size_t workspace_bytes, void *stream);
+
+/*
+ * Subsystem 4a — LRU lookup / touch / evict / slot-assign for one decode step.
+ * Replaces _update_page_access_time_, torch.argsort(page_access_time,
+ * stable=True) and the metadata half of _load_lru_cache_inline_kernel in
+ * dram_attention/lru_triton_kernel.py:6-194 (and current_step.add_(1),
+ * dram_attention/lru_cache.py:224, when `bump_step` is set).
+ *   idx          : (Hkv, K) requested DRAM pages in visiting order (itype idx_itype)
+ *   step         : one int32; with bump_step the kernel uses *step+1 and stores it
+ *   access_time  : (Hkv, N_hbm) last-use step per slot (fp32 or int32)
+ *   d2h          : (Hkv, P) slot of each DRAM page or -1;  h2d : (Hkv, N_hbm) page per slot
+ *                  (both of itype map_itype); updated in place
+ *   hit_mask     : optional (Hkv, K) bytes, 1 = page was resident when visited
+ *   miss_page/miss_slot : (Hkv, K) int32, the i-th distinct missed page of a
+ *                  head and the slot it was given; miss_count : (Hkv) int32
+ * The end state equals the reference's serial walk for every input; K <=
+ * N_hbm runs fully parallel, K > N_hbm falls back to one serial lane per head.
+ * A miss_slot of -1 marks an entry whose slot was re-assigned later in the
+ * same call (possible only when K > N_hbm); da_pages_gather skips it.
+ * workspace: da_lru_update_workspace_bytes(...) bytes, ZEROED ONCE by the
+ * caller before the first call and left alone afterwards.
+ */
+size_t da_lru_update_workspace_bytes(int n_kv_heads, int k, int64_t n_dram_pages,
+                                     int n_hbm_pages);
+int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_itype,
+                  int n_kv_heads, int k, int64_t n_dram_pages, int n_hbm_pages,
+                  int32_t *step, int bump_step, void *access_time,
+                  int64_t time_head_stride, int time_type, void *d2h,
+                  int64_t d2h_head_stride, void *h2d, int64_t h2d_head_stride,
+                  int map_itype, uint8_t *hit_mask, int32_t *miss_page,
+                  int32_t *miss_slot, int32_t *miss_count, void *workspace,
+                  size_t workspace_bytes, void *stream);
+
+/*
+ * Subsystem 4b — stream the missed pages into their HBM slots.
+ * Replaces the page copy loop of _load_lru_cache_inline_kernel,
+ * dram_attention/lru_triton_kernel.py:80-98 (8 serial programs reading host
+ * memory) by a grid-wide gather: every wave copies 16-byte lanes of one page.
+ *   dram : device-visible base of the (Hkv, P, page_bytes) page store
+ *   hbm  : base of the (Hkv, N_hbm, page_bytes) slot array
+ * Entry i < miss_count[h] of head h copies page miss_page[h,i] to slot
+ * miss_slot[h,i]; page_bytes must be a multiple of 16.
+ */
+int da_pages_gather(const void *dram, int64_t dram_head_stride_bytes,
+                    int64_t dram_page_stride_bytes, void *hbm,
+                    int64_t hbm_head_stride_bytes, int64_t hbm_slot_stride_bytes,
+                    int64_t page_bytes, const int32_t *miss_page,
+                    const int32_t *miss_slot, const int32_t *miss_count,
+                    int n_kv_heads, int k, void *stream);
+
+/*
+ * Subsystem 5 — split-K decode attention for ONE query token over
+ *   [prefix segment] ++ [local segment (c_len rows)] ++ [the new token],
+ * with the new key/value appended in place at row c_len of the local cache and
+ * all partial results merged through their log-sum-exp.  Replaces both
+ * flash_attn_with_kvcache calls and _combine_attention in
+ * dram_attention/dram_attention.py:191-238.
+ *   q            : (Hq, D), head stride q_head_stride; q head j uses kv head j / (Hq/Hkv)
+ *   pk, pv       : prefix keys / values, (Hkv, p_len, D) with element strides
+ *                  (p_head_stride, p_tok_stride, 1); p_len may be 0
+ *   ck, cv       : local cache, (capacity, Hkv, D) addressed with (c_tok_stride, c_head_stride, 1)
+ *   c_len        : rows already valid in the local cache; if c_len_dev is not
+ *                  NULL the value is read from that device int32 instead
+ *   new_k, new_v : (Hkv, D) of the current token (head stride new_head_stride),
+ *                  or NULL to attend over the c_len cached rows only
+ *   out          : (Hq, D) in `dtype`;  lse_out : optional (Hq) fp32, natural log
+ * fp32 accumulation throughout; 16-bit inputs use packed dot products, so
+ * probabilities are rounded to the input type before they weight the values
+ * (as flash-attn does).
+ */
+size_t da_decode_attention_workspace_bytes(int n_q_heads, int n_kv_heads, int head_dim,
+                                           int dtype, int64_t p_len, int64_t c_capacity);
+int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
+                        int n_kv_heads, int head_dim, int dtype, const void *pk,
+                        const void *pv, int64_t p_tok_stride, int64_t p_head_stride,
+                        int64_t p_len, void *ck, void *cv, int64_t c_tok_stride,
+                        int64_t c_head_stride, int64_t c_capacity, int64_t c_len,
+                        const int32_t *c_len_dev, const void *new_k, const void *new_v,
+                        int64_t new_head_stride, float scale, void *out,
+                        int64_t out_head_stride, float *lse_out, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DRAM_ATTENTION_AMD_H */

@@ -1,0 +1,346 @@
+"""Parity of every HIP kernel (called through the C ABI) against the CPU oracle."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dram_attention_oracle as O
+from tests.golden import lru_kats
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ------------------------------------------------------------------ page min/max
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("H,P,page,D", [(2, 5, 16, 64), (8, 33, 16, 128), (3, 7, 4, 24),
+                                        (2, 9, 8, 5), (1, 1, 1, 1)])
+def test_page_minmax_exact(dtype, H, P, page, D):
+    from dram_attention_amd.topk_selector import page_min_max
+
+    k = torch.randn(H, P * page, D, generator=gen(1)).to(dtype)
+    got = page_min_max(k.to(DEV), P)
+    assert torch.equal(got.cpu(), O.page_min_max(k, P))
+    # the layout init_cache hands over: a (S, H, D) tensor viewed as (H, S, D)
+    kt = k.transpose(0, 1).contiguous().to(DEV).transpose(0, 1)
+    assert not kt.is_contiguous() or H == 1 or P * page == 1
+    assert torch.equal(page_min_max(kt, P).cpu(), O.page_min_max(k, P))
+
+
+def test_page_minmax_nan_propagates():
+    from dram_attention_amd.topk_selector import page_min_max
+
+    k = torch.randn(1, 32, 8, generator=gen(2))
+    k[0, 5, 3] = float("nan")
+    got = page_min_max(k.to(DEV), 2).cpu()
+    assert torch.isnan(got[0, 0, :, 3]).all() and not torch.isnan(got[0, 1]).any()
+    assert not torch.isnan(got[0, 0, :, :3]).any()
+
+
+# ------------------------------------------------------------------ scorer
+def test_max_inner_product_reference_cases():
+    """The five cases of the reference's max_ip_triton_kernel_test.py."""
+    from dram_attention_amd import max_inner_product, max_ip_ref
+
+    q = torch.randn(2, 4, 64, generator=gen(3))
+    mm = torch.randn(4, 16, 2, 64, generator=gen(4))
+    out = max_inner_product(q.to(DEV), mm.to(DEV))
+    assert out.shape == (2, 4, 16) and out.dtype == torch.float32
+    assert torch.allclose(out.cpu(), O.max_ip(q, mm), rtol=1e-3, atol=1e-3)   # :29-38 tolerance
+    assert torch.allclose(out, max_ip_ref(q.to(DEV), mm.to(DEV)), rtol=1e-3, atol=1e-3)
+    out16 = max_inner_product(q.half().to(DEV), mm.half().to(DEV))
+    assert out16.dtype == torch.float16
+    q1, mm1 = torch.randn(1, 1, 1, generator=gen(5)), torch.randn(1, 1, 2, 1, generator=gen(6))
+    o1 = max_inner_product(q1.to(DEV), mm1.to(DEV))
+    assert o1.shape == (1, 1, 1)
+    assert o1.item() == pytest.approx(max(q1.item() * mm1[0, 0, 0, 0].item(),
+                                          q1.item() * mm1[0, 0, 1, 0].item()), rel=1e-6)
+    qL = torch.randn(32, 32, 128, generator=gen(7))
+    mmL = torch.randn(32, 1024, 2, 128, generator=gen(8))
+    oL = max_inner_product(qL.to(DEV), mmL.to(DEV))
+    assert oL.shape == (32, 32, 1024)
+    assert torch.allclose(oL.cpu(), O.max_ip(qL, mmL), rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("N,H,D,L", [(4, 8, 128, 515), (8, 2, 64, 130), (1, 3, 128, 4),
+                                     (5, 2, 40, 37), (3, 2, 256, 9)])
+def test_page_score_bf16_matches_reference_rounding(N, H, D, L):
+    from dram_attention_amd import max_inner_product
+
+    q = torch.randn(N, H, D, generator=gen(9)).bfloat16()
+    mm = torch.randn(H, L, 2, D, generator=gen(10)).bfloat16()
+    got = max_inner_product(q.to(DEV), mm.to(DEV)).cpu()
+    want = O.max_ip(q, mm)
+    assert got.dtype == torch.bfloat16
+    # same rounding points; fp32 summation order differs, so a sum that lands on a
+    # bf16 rounding boundary may fall to the neighbouring value: at most one ulp, rarely
+    diff = (got.float() - want.float()).abs()
+    ulp = want.float().abs() * 2.0 ** -7
+    assert torch.all(diff <= ulp + 1e-30)
+    assert (diff > 0).float().mean().item() < 0.02
+
+
+def test_page_score_strided_query_view():
+    """The (rep, Hkv, D) view of one token's query heads: strides (D, rep*D, 1)."""
+    from dram_attention_amd.max_ip_kernel import page_scores
+
+    Hkv, rep, D, L = 8, 4, 128, 300
+    q = torch.randn(1, 1, Hkv * rep, D, generator=gen(11)).bfloat16()
+    mm = torch.randn(Hkv, L, 2, D, generator=gen(12)).bfloat16()
+    qd = q.to(DEV)
+    qv = qd[0, 0].view(Hkv, rep, D).transpose(0, 1)
+    out = torch.empty(rep, Hkv, L, dtype=torch.float32, device=DEV)
+    page_scores(qv, mm.to(DEV), out, round_to_input=True)
+    want = O.scores_for_selection(q, mm)
+    diff = (out.cpu() - want).abs()
+    assert torch.all(diff <= want.abs() * 2.0 ** -7)
+    # fp32 output holds bf16-representable values
+    assert torch.equal(out.cpu(), out.cpu().bfloat16().float())
+
+
+# ------------------------------------------------------------------ top-k
+def run_topk(scores, rep, k):
+    from dram_attention_amd.topk_selector import topk_pages
+
+    n_rows, H, L = scores.shape
+    seq = n_rows // rep
+    out = torch.empty(seq, H, rep, k, dtype=torch.int64, device=DEV)
+    topk_pages(scores.to(DEV), rep, k, out, H * rep * k, rep * k, k)
+    return out.cpu()
+
+
+@pytest.mark.parametrize("rows,rep,H,L,k", [(4, 4, 8, 8192, 256), (2, 2, 2, 512, 32),
+                                            (3, 1, 2, 1000, 1000), (6, 3, 1, 77, 5),
+                                            (1, 1, 1, 1, 1), (2, 1, 2, 5000, 1),
+                                            (8, 8, 2, 20000, 512), (1, 1, 1, 300, 299)])
+def test_topk_pages_exact(rows, rep, H, L, k):
+    scores = torch.randn(rows, H, L, generator=gen(13))
+    got = run_topk(scores, rep, k)
+    want = O.select_pages(scores, rows // rep, rep, k)
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("levels", [2, 7, 200])
+def test_topk_pages_ties_lowest_index_first(levels):
+    scores = torch.randint(0, levels, (4, 4, 4096), generator=gen(14)).float() - levels / 2
+    got = run_topk(scores, 4, 256)
+    assert torch.equal(got, O.select_pages(scores, 1, 4, 256))
+    # bf16-rounded scores, the production case
+    s2 = (torch.randn(4, 8, 8192, generator=gen(15)) * 20).bfloat16().float()
+    assert torch.equal(run_topk(s2, 4, 256), O.select_pages(s2, 1, 4, 256))
+
+
+def test_topk_pages_special_values():
+    s = torch.randn(2, 1, 600, generator=gen(16))
+    s[0, 0, 10] = float("inf")
+    s[0, 0, 20] = -float("inf")
+    s[0, 0, 30] = 0.0
+    s[0, 0, 31] = -0.0
+    s[1, 0, :] = 1.5                      # one constant row: indices 0..k-1
+    s[1, 0, 100] = float("nan")           # torch ranks NaN first when descending
+    got = run_topk(s, 1, 300)
+    want = O.select_pages(s, 2, 1, 300)
+    assert torch.equal(got, want)
+    assert got[1, 0, 0, 0].item() == 100 and got[1, 0, 0, 1:5].tolist() == [0, 1, 2, 3]
+
+
+def test_topk_for_lru_layout():
+    from dram_attention_amd.topk_selector import topk_pages
+
+    seq, rep, H, L, k = 3, 2, 4, 200, 6
+    scores = torch.randn(seq * rep, H, L, generator=gen(17))
+    out = torch.empty(H, seq * rep * k, dtype=torch.int64, device=DEV)
+    topk_pages(scores.to(DEV), rep, k, out, rep * k, seq * rep * k, k)
+    want = O.lru_index_list(O.select_pages(scores, seq, rep, k))
+    assert torch.equal(out.cpu(), want)
+    out32 = torch.empty(H, seq * rep * k, dtype=torch.int32, device=DEV)
+    topk_pages(scores.to(DEV), rep, k, out32, rep * k, seq * rep * k, k)
+    assert torch.equal(out32.cpu().long(), want)
+
+
+# ------------------------------------------------------------------ LRU
+@pytest.mark.parametrize("name", sorted(lru_kats.CASES))
+def test_load_lru_cache_reference_kats(name):
+    from dram_attention_amd import load_lru_cache_
+
+    case = lru_kats.CASES[name]
+    H, P, N, PD = (lru_kats.NUM_HEADS, lru_kats.NUM_DRAM_PAGES, lru_kats.NUM_HBM_PAGES,
+                   lru_kats.PAGE_DIM)
+    dram = torch.randn(H, P, PD, generator=gen(18)).to(DEV)
+    hbm = torch.zeros(H, N, PD, device=DEV)
+    time = torch.arange(N, dtype=torch.int32, device=DEV).repeat(H, 1)
+    d2h = torch.tensor(case["d2h"], dtype=torch.int32, device=DEV)
+    h2d = torch.tensor(case["h2d"], dtype=torch.int32, device=DEV)
+    for h in range(H):
+        for s, p in enumerate(case["h2d"][h]):
+            if p >= 0:
+                hbm[h, s] = dram[h, p]
+    topk = torch.tensor(case["topk"], dtype=torch.int32, device=DEV)
+    step = torch.tensor([lru_kats.STEP], dtype=torch.int32, device=DEV)
+    load_lru_cache_(dram_kv_cache=dram, page_access_time=time,
+                    dram_page_to_hbm_page_mapping=d2h, hbm_page_to_dram_page_mapping=h2d,
+                    topk_dram_page_index=topk, current_step=step, hbm_kv_cache=hbm)
+    for (h, s), t in case["time"].items():
+        assert time[h, s].item() == t
+    for (h, p), s in case["d2h_after"].items():
+        assert d2h[h, p].item() == s
+    for (h, s), p in case["h2d_after"].items():
+        assert h2d[h, s].item() == p
+    for h, s, p in case["payload"]:
+        assert torch.equal(hbm[h, s], dram[h, p])
+    assert step.item() == lru_kats.STEP        # the raw function does not advance the step
+
+
+def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat16, page_dim=256,
+              hot=None):
+    """Random request trace on LRUCache-like state; compares every buffer with the
+    oracle's serial walk after every step."""
+    from dram_attention_amd.lru_kernel import LruScratch, lru_update_and_gather
+
+    rng = np.random.default_rng(seed)
+    dram = torch.randn(H, P, page_dim, generator=gen(seed)).to(dtype)
+    dram_dev = dram.pin_memory() if pinned else dram.to(DEV)
+    st = O.LruState.initial(H, P, N)
+    hbm_o = dram[:, P - N:].clone()
+    hbm = hbm_o.to(DEV)
+    time = torch.zeros(H, N, dtype=ttype, device=DEV)
+    d2h = torch.from_numpy(st.d2h).to(itype).to(DEV)
+    h2d = torch.from_numpy(st.h2d).to(itype).to(DEV)
+    step = torch.zeros(1, dtype=torch.int32, device=DEV)
+    scratch = LruScratch.allocate(H, K, DEV)
+    as_np = (lambda t: t.view(torch.int16).numpy()) if dtype != torch.float32 else (lambda t: t.numpy())
+    for s in range(1, steps + 1):
+        if hot:  # skewed requests with duplicates, like overlapping per-head top-k lists
+            idx = np.where(rng.random((H, K)) < 0.7, rng.integers(0, hot, (H, K)),
+                           rng.integers(0, P, (H, K)))
+        else:
+            idx = rng.integers(0, P, (H, K))
+        hit_o, miss_o = O.lru_load(st, idx, s, as_np(dram), as_np(hbm_o))
+        lru_update_and_gather(dram_dev, time, d2h, h2d, torch.from_numpy(idx).to(itype).to(DEV),
+                              step, hbm, scratch, bump_step=True)
+        torch.cuda.synchronize()
+        assert step.item() == s
+        assert np.array_equal(time.cpu().numpy().astype(np.float32), st.time), f"time, step {s}"
+        assert np.array_equal(d2h.cpu().numpy(), st.d2h), f"d2h, step {s}"
+        assert np.array_equal(h2d.cpu().numpy(), st.h2d), f"h2d, step {s}"
+        assert np.array_equal(scratch.hit_mask.cpu().numpy().astype(bool), hit_o), f"hits, step {s}"
+        counts = scratch.miss_count.cpu().tolist()
+        mp, ms = scratch.miss_page.cpu().numpy(), scratch.miss_slot.cpu().numpy()
+        for h in range(H):
+            assert counts[h] == len(miss_o[h])
+            got = [(int(mp[h, i]), int(ms[h, i])) for i in range(counts[h])]
+            if K <= N:
+                assert got == miss_o[h]
+            else:  # serial walk: entries overwritten later in the call are marked dead
+                live = {}
+                for p, v in miss_o[h]:
+                    live[v] = p
+                assert [(p, v) for p, v in got if v >= 0] == \
+                    [(p, v) for p, v in miss_o[h] if live[v] == p]
+        assert torch.equal(hbm.cpu(), hbm_o), f"payload, step {s}"
+
+
+@pytest.mark.parametrize("H,P,N,K,itype,ttype,pinned", [
+    (2, 64, 16, 8, torch.int64, torch.float32, True),
+    (8, 512, 128, 128, torch.int64, torch.float32, True),      # K == N_hbm
+    (3, 300, 100, 37, torch.int32, torch.int32, False),
+    (4, 2048, 1024, 1024, torch.int64, torch.float32, False),  # K == N_hbm, several scan rounds
+    (2, 4096, 2048, 1500, torch.int64, torch.float32, True),
+])
+def test_lru_update_matches_serial_walk(H, P, N, K, itype, ttype, pinned):
+    lru_trace(H, P, N, K, 12, 100 + K, itype, ttype, pinned)
+    lru_trace(H, P, N, K, 12, 200 + K, itype, ttype, pinned, hot=max(2, P // 8))
+
+
+@pytest.mark.parametrize("H,P,N,K", [(2, 40, 6, 17), (1, 8, 2, 3), (3, 200, 50, 120)])
+def test_lru_update_more_requests_than_slots(H, P, N, K):
+    lru_trace(H, P, N, K, 8, 300 + K, torch.int64, torch.float32, False, dtype=torch.float32,
+              page_dim=32)
+    lru_trace(H, P, N, K, 8, 400 + K, torch.int64, torch.float32, False, dtype=torch.float32,
+              page_dim=32, hot=max(2, P // 4))
+
+
+# ------------------------------------------------------------------ decode attention
+def dense_reference(q, segments):
+    k = torch.cat([s[0] for s in segments], dim=1)
+    v = torch.cat([s[1] for s in segments], dim=1)
+    return O.attention_partial(q, k, v)
+
+
+@pytest.mark.parametrize("dtype,atol,rtol", [(torch.float32, 2e-5, 1e-4),
+                                             (torch.bfloat16, 2e-2, 1e-2),
+                                             (torch.float16, 4e-3, 1e-2)])
+@pytest.mark.parametrize("Hq,Hkv,D,p_len,c_len,cap", [
+    (32, 8, 128, 2048, 500, 640), (8, 2, 64, 512, 1008, 1040), (4, 4, 128, 0, 77, 128),
+    (16, 2, 64, 333, 0, 64), (6, 2, 128, 1000, 31, 32), (2, 1, 256, 40, 3, 8),
+    (64, 8, 128, 4096, 100, 200)])
+def test_decode_attention_matches_dense(dtype, atol, rtol, Hq, Hkv, D, p_len, c_len, cap):
+    from dram_attention_amd import decode_attention
+
+    g = gen(19)
+    q = torch.randn(Hq, D, generator=g).to(dtype)
+    # the prefix as the LRU hands it over: K/V interleaved per token
+    inter = torch.randn(Hkv, max(p_len, 1), 2, D, generator=g).to(dtype)[:, :p_len]
+    ck = torch.zeros(cap, Hkv, D, dtype=dtype)
+    cv = torch.zeros(cap, Hkv, D, dtype=dtype)
+    ck[:c_len] = torch.randn(c_len, Hkv, D, generator=g).to(dtype)
+    cv[:c_len] = torch.randn(c_len, Hkv, D, generator=g).to(dtype)
+    nk = torch.randn(Hkv, D, generator=g).to(dtype)
+    nv = torch.randn(Hkv, D, generator=g).to(dtype)
+    want, want_lse = dense_reference(q, [
+        (inter[:, :, 0], inter[:, :, 1]),
+        (ck[:c_len].transpose(0, 1), cv[:c_len].transpose(0, 1)),
+        (nk[:, None], nv[:, None])])
+    inter_d, ckd, cvd = inter.to(DEV), ck.to(DEV), cv.to(DEV)
+    lse = torch.empty(Hq, dtype=torch.float32, device=DEV)
+    out = decode_attention(q.to(DEV), inter_d[:, :, 0], inter_d[:, :, 1], ckd, cvd, c_len,
+                           nk.to(DEV), nv.to(DEV), lse=lse)
+    assert out.dtype == dtype
+    assert torch.allclose(out.cpu().float(), want, atol=atol, rtol=rtol)
+    assert torch.allclose(lse.cpu(), want_lse, atol=2e-3 if dtype != torch.float32 else 1e-4)
+    # the append happened in place, nothing else moved
+    assert torch.equal(ckd[c_len].cpu(), nk) and torch.equal(cvd[c_len].cpu(), nv)
+    assert torch.equal(ckd[:c_len].cpu(), ck[:c_len]) and torch.equal(ckd[c_len + 1:].cpu(), ck[c_len + 1:])
+    # device-side length gives the same bits
+    ckd2, cvd2 = ck.to(DEV), cv.to(DEV)
+    out2 = decode_attention(q.to(DEV), inter_d[:, :, 0], inter_d[:, :, 1], ckd2, cvd2,
+                            torch.tensor([c_len], dtype=torch.int32, device=DEV),
+                            nk.to(DEV), nv.to(DEV))
+    assert torch.equal(out2, out) and torch.equal(ckd2, ckd)
+
+
+def test_decode_attention_large_logits_and_no_append():
+    from dram_attention_amd import decode_attention
+
+    g = gen(20)
+    Hq, Hkv, D, T = 8, 2, 128, 700
+    q = (torch.randn(Hq, D, generator=g) * 6).bfloat16()
+    k = (torch.randn(Hkv, T, D, generator=g) * 3).bfloat16()
+    v = torch.randn(Hkv, T, D, generator=g).bfloat16()
+    ck = k[:, 400:].transpose(0, 1).contiguous()
+    cv = v[:, 400:].transpose(0, 1).contiguous()
+    out = decode_attention(q.to(DEV), k[:, :400].to(DEV), v[:, :400].to(DEV), ck.to(DEV),
+                           cv.to(DEV), 300, None, None)
+    want, _ = O.attention_partial(q, k, v)
+    assert torch.allclose(out.cpu().float(), want, atol=2e-2, rtol=1e-2)
+
+
+def test_decode_attention_rejects_overflow_and_bad_dim():
+    from dram_attention_amd import decode_attention
+
+    q = torch.zeros(4, 64, device=DEV)
+    c = torch.zeros(8, 2, 64, device=DEV)
+    n = torch.zeros(2, 64, device=DEV)
+    with pytest.raises(RuntimeError, match="overflow"):
+        decode_attention(q, None, None, c, c.clone(), 8, n, n)
+    with pytest.raises(RuntimeError):
+        decode_attention(torch.zeros(4, 24, device=DEV), None, None,
+                         torch.zeros(8, 2, 24, device=DEV), torch.zeros(8, 2, 24, device=DEV), 1,
+                         None, None)

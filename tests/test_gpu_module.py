@@ -1,0 +1,286 @@
+"""The drop-in surface (LRUCache, DRAMAttention) on the GPU: the reference's own
+object-level tests restated, and step-by-step parity of whole decode runs with
+the CPU oracle."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from dram_attention_amd.synthetic import WORKLOADS, DecodeInputs, make_prompt
+from oracle import dram_attention_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+# ------------------------------------------------------------ reference lru_cache_test.py
+@pytest.fixture
+def sample_cache():
+    from dram_attention_amd import LRUCache
+
+    g = torch.Generator().manual_seed(0)
+    k = torch.randn(4, 1024 * 8, 64, generator=g).to(DEV)
+    v = torch.randn(4, 1024 * 8, 64, generator=g).to(DEV)
+    return LRUCache(k, v, page_size=16, top_k=10)
+
+
+def test_lru_cache_initialization(sample_cache):
+    c = sample_cache
+    assert (c.num_kv_heads, c.num_dram_pages, c.num_hbm_pages) == (4, 512, 102)
+    assert (c.head_dim, c.page_size, c.top_k) == (64, 16, 10)
+    assert torch.all(c.dram_page_to_hbm_page_mapping[:, -102:] == torch.arange(102, device=DEV))
+    assert torch.all(c.dram_page_to_hbm_page_mapping[:, :-102] == -1)
+    assert c.dram_kv_cache.is_pinned() and c.dram_kv_cache.shape == (4, 512, 16 * 2 * 64)
+    assert torch.equal(c.hbm_kv_cache.cpu(), c.dram_kv_cache[:, -102:])
+
+
+def test_lru_cache_load_inline_method(sample_cache):
+    idx = torch.randint(0, 512, (4, 10), device=DEV)
+    k_cache, v_cache = sample_cache.load_(idx)
+    assert k_cache.shape == (4, 102 * 16, 64) and v_cache.shape == (4, 102 * 16, 64)
+    assert sample_cache.current_step == 1
+    # every requested page is resident and its payload sits in the slot the map names
+    slots = torch.gather(sample_cache.dram_page_to_hbm_page_mapping, 1, idx)
+    assert torch.all(slots >= 0)
+    for h in range(4):
+        got = sample_cache.hbm_kv_cache[h, slots[h]].cpu()
+        assert torch.equal(got, sample_cache.dram_kv_cache[h, idx[h].cpu()])
+
+
+@pytest.mark.parametrize("page_size", [8, 16, 32])
+def test_lru_cache_different_page_sizes(page_size):
+    from dram_attention_amd import LRUCache
+
+    k = torch.randn(4, 1024 * 8, 64)
+    v = torch.randn(4, 1024 * 8, 64)
+    cache = LRUCache(k, v, page_size=page_size, top_k=10)     # host tensors are accepted
+    assert cache.page_size == page_size and cache.num_dram_pages == 1024 * 8 // page_size
+    assert cache.top_k == 10
+    assert cache.top_k_selector.chunk_min_max.shape == (4, 1024 * 8 // page_size, 2, 64)
+
+
+def test_lru_cache_invalid_initialization_and_hbm_size():
+    from dram_attention_amd import LRUCache
+
+    with pytest.raises(AssertionError):
+        LRUCache(torch.randn(4, 1007 * 8, 64), torch.randn(4, 1007 * 8, 64), page_size=16, top_k=10)
+    k = torch.randn(4, 1024 * 8, 64)
+    cache = LRUCache(k, k.clone(), page_size=16, lru_hbm_cache_size=1024, top_k=10)
+    assert cache.num_hbm_pages == 64 and cache.top_k == 10
+
+
+def test_lru_cache_get_kv_cache_inline(sample_cache):
+    query = torch.randn(1, 10, 4, 64, generator=torch.Generator().manual_seed(1)).to(DEV)
+    out = sample_cache.get_kv_cache_(query)
+    assert out.k_cache.shape == (4, 102 * 16, 64) and out.v_cache.shape == (4, 102 * 16, 64)
+    assert sample_cache.current_step == 1
+    sample_cache.get_kv_cache_(query)
+    assert sample_cache.current_step == 2
+    assert out.k_cache.device.type == "cuda" and out.v_cache.device.type == "cuda"
+    assert torch.any(out.k_cache != 0) and torch.any(out.v_cache != 0)
+    # selection of a 10-token query block equals the oracle's on the kernel's own scores
+    sel = sample_cache.top_k_selector
+    scores = sel.scores(query).cpu()
+    want = O.select_pages(scores, 10, 1, 10)
+    assert torch.equal(sel.top_k(query, 10).cpu(), want)
+
+
+# ------------------------------------------------------------ reference dram_attention_test.py
+def make_module(**kw):
+    from dram_attention_amd import DRAMAttention
+
+    args = dict(max_output_length=64, lru_hbm_cache_size=32 * 1024, local_cache_size=4096 + 512,
+                page_size=16, top_k=4096, n_kv_heads=8, head_dim=128, device=DEV)
+    args.update(kw)
+    return DRAMAttention(**args)
+
+
+def test_module_init_and_errors():
+    m = make_module()
+    assert (m.max_output_length, m.lru_hbm_cache_size, m.local_cache_size) == (64, 32768, 4608)
+    assert (m.page_size, m.top_k, m.n_kv_heads, m.head_dim) == (16, 4096, 8, 128)
+    assert m.cache_k.shape == (1, 4608 + 64, 8, 128) and m.cache_k.dtype == torch.bfloat16
+    x = torch.randn(1, 1, 8, 128, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="Unsupported stage"):
+        m(x, x, x, start_pos=0, stage="invalid")
+    x2 = torch.randn(2, 1, 8, 128, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="Only support batch size 1"):
+        m(x2, x2, x2, start_pos=0, stage="prefill")
+
+
+def test_module_prefill_then_generate_shapes():
+    """The reference's prefill/generate smoke at its 66K-token shape."""
+    m = make_module()
+    S = 66 * 1024
+    g = torch.Generator(device=DEV).manual_seed(0)
+    xq = torch.randn(1, S, 32, 128, device=DEV, dtype=torch.bfloat16, generator=g)
+    xk = torch.randn(1, S, 8, 128, device=DEV, dtype=torch.bfloat16, generator=g)
+    xv = torch.randn(1, S, 8, 128, device=DEV, dtype=torch.bfloat16, generator=g)
+    out = m(xq, xk, xv, start_pos=0, stage="prefill")
+    assert out.shape == (1, S, 32, 128)
+    assert m.dram_kv_cache_size == (S - 4608 + 16) // 16 * 16
+    # causal check on a few rows against a direct softmax
+    for row in (0, 17, 5000):
+        qs = xq[0, row].float().view(8, 4, 128)
+        s = torch.einsum("hrd,thd->hrt", qs, xk[0, : row + 1].float()) / math.sqrt(128)
+        want = torch.einsum("hrt,thd->hrd", torch.softmax(s, -1), xv[0, : row + 1].float())
+        assert torch.allclose(out[0, row].float().view(8, 4, 128), want, atol=2e-2, rtol=2e-2)
+    q1 = torch.randn(1, 1, 32, 128, device=DEV, dtype=torch.bfloat16, generator=g)
+    k1 = torch.randn(1, 1, 8, 128, device=DEV, dtype=torch.bfloat16, generator=g)
+    v1 = torch.randn(1, 1, 8, 128, device=DEV, dtype=torch.bfloat16, generator=g)
+    o1 = m(q1, k1, v1, start_pos=S, stage="generate")
+    assert o1.shape == (1, 1, 32, 128) and torch.isfinite(o1.float()).all()
+
+
+# ------------------------------------------------------------ whole decode runs vs the oracle
+def run_parity(w, seed, steps, atol, rtol, device_pos=False):
+    """Drives the module and the oracle with the same inputs.  Selection and LRU
+    state are compared bit for bit at every step, the oracle being fed the
+    kernel's scores (the contract is 'given identical scores'); the kernel's
+    scores themselves are compared with the oracle's within one rounding step."""
+    from dram_attention_amd import DRAMAttention, LRUCache
+
+    prompt = make_prompt(w, seed)
+    m = DRAMAttention(max_output_length=w.steps, lru_hbm_cache_size=w.lru_tokens,
+                      local_cache_size=w.local_cache, page_size=w.page_size,
+                      top_k=w.top_k_tokens, n_kv_heads=w.n_kv_heads, head_dim=w.head_dim,
+                      device=DEV, dtype=w.dtype)
+    m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+    o = O.DecodeOracle(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                       w.n_kv_heads, w.head_dim, dtype=w.dtype)
+    o.init_cache(prompt.k, prompt.v)
+    assert m.dram_kv_cache_size == o.dram_kv_cache_size == w.dram_tokens
+    assert isinstance(m.lru_cache, LRUCache) and o.uses_lru
+    lru = m.lru_cache
+    assert torch.equal(lru.top_k_selector.chunk_min_max.cpu(), o.min_max)
+    assert torch.equal(lru.dram_kv_cache, o.dram)
+    inputs = DecodeInputs(w, prompt.q0, seed)
+    pos = torch.tensor([w.prompt_tokens], dtype=torch.int32, device=DEV)
+    hits = total = 0
+    for t in range(steps):
+        xq, xk, xv = inputs.next()
+        start = w.prompt_tokens + t
+        out = m(xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=pos if device_pos else start,
+                stage="generate")
+        pos += 1
+        scores = lru.top_k_selector._scores.cpu()
+        own = O.scores_for_selection(xq, o.min_max)
+        assert torch.all((scores - own).abs() <= own.abs() * 2.0 ** -7 + 1e-4), f"scores, step {t}"
+        want = o.generate(xq, xk, xv, start, scores=scores)
+        assert torch.equal(lru._topk_idx.cpu(), o.last_idx), f"selection, step {t}"
+        if t == 0:
+            for h, page in prompt.planted:
+                assert (o.last_idx[h] == page).any(), "planted page not selected"
+        assert lru.current_step.item() == o.state.step == t + 1
+        assert np.array_equal(lru.page_access_time.cpu().numpy(), o.state.time), f"time, step {t}"
+        assert np.array_equal(lru.dram_page_to_hbm_page_mapping.cpu().numpy(), o.state.d2h)
+        assert np.array_equal(lru.hbm_page_to_dram_page_mapping.cpu().numpy(), o.state.h2d)
+        assert np.array_equal(lru._scratch.hit_mask.cpu().numpy().astype(bool), o.last_hit)
+        assert torch.equal(lru.hbm_kv_cache.cpu(), o.hbm), f"slot payload, step {t}"
+        assert torch.allclose(out.cpu().float(), want.float(), atol=atol, rtol=rtol), f"output, step {t}"
+        hits += int(o.last_hit.sum())
+        total += o.last_hit.size
+    c = w.prompt_tokens + steps - w.dram_tokens
+    assert torch.equal(m.cache_k[0, :c].cpu(), o.cache_k[:c])
+    assert torch.equal(m.cache_v[0, :c].cpu(), o.cache_v[:c])
+    return hits / total
+
+
+def test_decode_parity_cpu_reference_config():
+    """configs[0] exactly: fp32, 8/2 heads, D 64, 8192-token prefix, K == N_hbm."""
+    w = WORKLOADS["cpu"]
+    rate = run_parity(w, 0, w.steps, atol=1e-4, rtol=1e-4)
+    assert 0.0 < rate < 1.0
+
+
+def test_decode_parity_bf16_scaled_llama_shape():
+    """The 128K layer shape scaled to a prefix the oracle walks in seconds."""
+    w = WORKLOADS["128k"].scaled(dram_tokens=16384, local_cache=1024, lru_tokens=4096,
+                                 top_k_tokens=1024, steps=12)
+    run_parity(w, 1, w.steps, atol=2e-2, rtol=1e-2)
+
+
+def test_decode_parity_device_side_position_and_rep8():
+    w = WORKLOADS["1m"].scaled(dram_tokens=8192, local_cache=512, lru_tokens=2048,
+                               top_k_tokens=256, steps=6, planted_pages=8)
+    run_parity(w, 2, w.steps, atol=2e-2, rtol=1e-2, device_pos=True)
+
+
+def test_static_prefix_equals_full_attention():
+    """Prefix within the HBM budget: the static cache path is dense attention over
+    the whole sequence (the 32K configuration through init_cache)."""
+    from dram_attention_amd import DRAMAttention, DummyCache
+
+    w = WORKLOADS["32k"].scaled(dram_tokens=4096, local_cache=512, lru_tokens=4096, steps=3)
+    prompt = make_prompt(w, 3)
+    m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, 16, w.top_k_tokens, w.n_kv_heads,
+                      w.head_dim, device=DEV, dtype=w.dtype)
+    m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+    assert isinstance(m.lru_cache, DummyCache)
+    inputs = DecodeInputs(w, prompt.q0, 3)
+    ks, vs = [prompt.k[0]], [prompt.v[0]]
+    for t in range(w.steps):
+        xq, xk, xv = inputs.next()
+        out = m(xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=w.prompt_tokens + t, stage="generate")
+        ks.append(xk[0]); vs.append(xv[0])
+        want, _ = O.attention_partial(xq[0, 0], torch.cat(ks).transpose(0, 1),
+                                      torch.cat(vs).transpose(0, 1))
+        assert torch.allclose(out[0, 0].cpu().float(), want, atol=2e-2, rtol=1e-2)
+
+
+# ------------------------------------------------------------ full size, by properties
+def test_headline_size_invariants():
+    """configs[2] (128K prefix, 8192 pages/head) at full size: invariants that need
+    no CPU walk, plus attention against a dense fp32 computation on the GPU."""
+    from dram_attention_amd import DRAMAttention
+
+    w = WORKLOADS["128k"]
+    prompt = make_prompt(w, 0)
+    m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, 16, w.top_k_tokens, w.n_kv_heads,
+                      w.head_dim, device=DEV, dtype=w.dtype)
+    m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+    lru = m.lru_cache
+    dram_dev = lru.dram_kv_cache.to(DEV)
+    inputs = DecodeInputs(w, prompt.q0, 0)
+    N, P = w.n_hbm_pages, w.n_dram_pages
+    ar = torch.arange(N, device=DEV)
+    for t in range(6):
+        xq, xk, xv = inputs.next()
+        xq, xk, xv = xq.to(DEV), xk.to(DEV), xv.to(DEV)
+        out = m(xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
+        idx, d2h, h2d = lru._topk_idx, lru.dram_page_to_hbm_page_mapping, lru.hbm_page_to_dram_page_mapping
+        assert idx.shape == (8, 1024)
+        # selection: sorted by (score desc, index asc) within each query head, and no
+        # unselected page beats the last selected one
+        scores = lru.top_k_selector._scores                         # (rep, H, P)
+        sel = idx.view(8, 4, 256)
+        s_sel = torch.gather(scores.transpose(0, 1), 2, sel)          # (H, rep, 256)
+        assert torch.all((s_sel[..., :-1] > s_sel[..., 1:]) |
+                         ((s_sel[..., :-1] == s_sel[..., 1:]) & (sel[..., :-1] < sel[..., 1:])))
+        mask = torch.ones(8, 4, P, dtype=torch.bool, device=DEV).scatter_(2, sel, False)
+        rest = scores.transpose(0, 1).masked_fill(~mask, -float("inf"))
+        best_rest, best_idx = rest.max(dim=-1)
+        last, last_idx = s_sel[..., -1], sel[..., -1]
+        assert torch.all((best_rest < last) | ((best_rest == last) & (best_idx > last_idx)))
+        # LRU maps: inverse of each other, all requests resident and touched now
+        assert torch.equal(torch.gather(d2h, 1, h2d), ar.expand(8, N))
+        assert (d2h >= 0).sum().item() == 8 * N
+        slots = torch.gather(d2h, 1, idx)
+        assert torch.all(slots >= 0)
+        assert torch.all(torch.gather(lru.page_access_time, 1, slots) == t + 1)
+        assert lru.current_step.item() == t + 1
+        # payload: every slot holds exactly the page the map names
+        want_pages = torch.gather(dram_dev, 1, h2d[:, :, None].expand(-1, -1, dram_dev.shape[2]))
+        assert torch.equal(lru.hbm_kv_cache, want_pages)
+        # attention over all resident slots ++ local window ++ new token
+        c = w.prompt_tokens + t - w.dram_tokens
+        kk = torch.cat([lru.hbm_kv_cache.view(8, N * 16, 2, 128)[:, :, 0],
+                        m.cache_k[0, : c + 1].transpose(0, 1)], 1).float()
+        vv = torch.cat([lru.hbm_kv_cache.view(8, N * 16, 2, 128)[:, :, 1],
+                        m.cache_v[0, : c + 1].transpose(0, 1)], 1).float()
+        s = torch.einsum("hrd,htd->hrt", xq[0, 0].float().view(8, 4, 128), kk) / math.sqrt(128)
+        want = torch.einsum("hrt,htd->hrd", torch.softmax(s, -1), vv).reshape(32, 128)
+        assert torch.allclose(out[0, 0].float(), want, atol=2e-2, rtol=1e-2)
+        assert torch.equal(m.cache_k[0, c], xk[0, 0]) and torch.equal(m.cache_v[0, c], xv[0, 0])

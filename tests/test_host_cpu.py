@@ -1,0 +1,120 @@
+"""CPU-side checks: the C-ABI library loads and exports every declared symbol,
+host-side argument checking, synthetic workloads, and that nothing computes
+without the GPU (the HIP kernels are the only implementation)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "dram_attention_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(da_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from dram_attention_amd import _lib
+
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 12
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == names        # the binding covers the header exactly
+    assert lib.da_version() >= 100
+    assert lib.da_last_error_string() is not None
+
+
+def test_workspace_queries_need_no_gpu(lib):
+    n = lib.da_decode_attention_workspace_bytes(32, 8, 128, 2, 32768, 4160)
+    assert n > 32 * 130 * 4
+    assert lib.da_decode_attention_workspace_bytes(32, 8, 24, 2, 1024, 64) == 0   # unsupported dim
+    assert lib.da_lru_update_workspace_bytes(8, 1024, 8192, 2048) >= 4
+
+
+def test_argument_checks_reject_before_any_launch(lib):
+    # null pointers / bad geometry are refused on the host: no GPU is touched
+    assert lib.da_page_score(None, 0, 0, None, 0, 0, 0, 4, 8, 16, 128, 2, None, 0, 0, 0, 1, None) == -1
+    assert b"null" in lib.da_last_error_string()
+    assert lib.da_page_score(None, 0, 0, None, 0, 0, 0, 4, 8, 16, 128, 9, None, 0, 0, 0, 1, None) == -1
+    assert lib.da_topk_pages(None, 0, 0, 1, 1, 1, 10, 11, None, 0, 0, 0, 1, None, 0, None) == -1
+    assert b"exceeds" in lib.da_last_error_string()
+    assert lib.da_pages_gather(ctypes.c_void_p(16), 0, 0, ctypes.c_void_p(16), 0, 0, 24,
+                               ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16),
+                               1, 1, None) == -1
+
+
+def test_module_surface_and_errors_on_cpu():
+    from dram_attention_amd import DRAMAttention
+
+    m = DRAMAttention(max_output_length=64, lru_hbm_cache_size=32 * 1024,
+                      local_cache_size=4096 + 512, page_size=16, top_k=4096, n_kv_heads=8,
+                      head_dim=128, device="cpu")
+    assert m.num_page == 2048 and m.dram_kv_cache_size is None
+    assert m.cache_k.shape == (1, 4096 + 512 + 64, 8, 128) and m.cache_v.dtype == torch.bfloat16
+    assert set(m.state_dict()) == {"cache_k", "cache_v"}
+    x = torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="Unsupported stage"):
+        m(x, x, x, start_pos=0, stage="invalid")
+    x2 = torch.zeros(2, 1, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="Only support batch size 1"):
+        m(x2, x2, x2, start_pos=0, stage="prefill")
+
+
+def test_no_cpu_fallback():
+    from dram_attention_amd import LRUCache, max_inner_product
+
+    with pytest.raises(RuntimeError, match="GPU"):
+        max_inner_product(torch.zeros(2, 4, 64), torch.zeros(4, 16, 2, 64))
+    with pytest.raises(RuntimeError, match="GPU"):
+        LRUCache(torch.zeros(2, 64, 8), torch.zeros(2, 64, 8), page_size=16, top_k=2, device="cpu")
+    with pytest.raises(AssertionError):
+        LRUCache(torch.zeros(2, 60, 8), torch.zeros(2, 60, 8), page_size=16, top_k=2)
+
+
+def test_package_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "dram_attention_amd")
+    for name in os.listdir(pkg):
+        if name.endswith(".py"):
+            assert "oracle" not in open(os.path.join(pkg, name)).read(), name
+
+
+def test_max_ip_ref_formula():
+    from dram_attention_amd import max_ip_ref
+    from oracle import dram_attention_oracle as O
+
+    g = torch.Generator().manual_seed(0)
+    q, mm = torch.randn(2, 4, 64, generator=g), torch.randn(4, 16, 2, 64, generator=g)
+    assert torch.allclose(max_ip_ref(q, mm), O.max_ip(q, mm), atol=1e-4)
+
+
+def test_synthetic_workloads():
+    from dram_attention_amd.synthetic import WORKLOADS, DecodeInputs, make_prompt
+    from oracle import dram_attention_oracle as O
+
+    w = WORKLOADS["128k"]
+    assert (w.n_dram_pages, w.n_hbm_pages, w.pages_per_q_head, w.rep) == (8192, 2048, 256, 4)
+    assert O.dram_split(w.prompt_tokens, w.local_cache, w.page_size) == w.dram_tokens
+    w5 = WORKLOADS["1m"]
+    assert (w5.n_dram_pages, w5.n_hbm_pages, w5.pages_per_q_head * w5.rep) == (65536, 4096, 4096)
+    c = WORKLOADS["cpu"]
+    p1, p2 = make_prompt(c, 0), make_prompt(c, 0)
+    assert torch.equal(p1.k, p2.k) and p1.k.shape == (1, c.prompt_tokens, 2, 64)
+    assert len(p1.planted) == 4 and all(pg < c.n_dram_pages - c.n_hbm_pages for _, pg in p1.planted)
+    # planted pages top the oracle's ranking for their kv group at step 0
+    xq, xk, xv = DecodeInputs(c, p1.q0, 0).next()
+    mm = O.page_min_max(p1.k[0, : c.dram_tokens].transpose(0, 1), c.n_dram_pages)
+    idx = O.lru_index_list(O.select_pages(O.scores_for_selection(xq, mm), 1, c.rep,
+                                          c.pages_per_q_head))
+    for h, page in p1.planted:
+        assert (idx[h] == page).any()
+    a, b = DecodeInputs(c, p1.q0, 0), DecodeInputs(c, p1.q0, 0)
+    for _ in range(3):
+        for x, y in zip(a.next(), b.next()):
+            assert torch.equal(x, y)
