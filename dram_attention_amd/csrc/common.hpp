@@ -56,6 +56,12 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
+// Reinterpreting helpers take their operand BY VALUE: __builtin_bit_cast applied
+// directly to a vector subscript (v[i]) reads element 0 with this compiler.
+__device__ __forceinline__ float as_f32(uint32_t w) { return __builtin_bit_cast(float, w); }
+__device__ __forceinline__ bf16x2 as_bf16x2(uint32_t w) { return __builtin_bit_cast(bf16x2, w); }
+__device__ __forceinline__ f16x2 as_f16x2(uint32_t w) { return __builtin_bit_cast(f16x2, w); }
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) {
   return __builtin_bit_cast(float, bits16 << 16);
 }
@@ -133,7 +139,7 @@ __device__ __forceinline__ void unpack(const u32x4 &v, float *f);
 template <>
 __device__ __forceinline__ void unpack<F32>(const u32x4 &v, float *f) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) f[i] = __builtin_bit_cast(float, v[i]);
+  for (int i = 0; i < 4; ++i) f[i] = as_f32(v[i]);
 }
 template <>
 __device__ __forceinline__ void unpack<F16>(const u32x4 &v, float *f) {

@@ -37,7 +37,7 @@ __device__ __forceinline__ float dot16<F32>(const u32x4 &q, const u32x4 &k) {
   float a = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
-    a = fmaf(__builtin_bit_cast(float, q[i]), __builtin_bit_cast(float, k[i]), a);
+    a = fmaf(as_f32(q[i]), as_f32(k[i]), a);
   return a;
 }
 template <>
@@ -45,8 +45,7 @@ __device__ __forceinline__ float dot16<BF16>(const u32x4 &q, const u32x4 &k) {
   float a = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
-    a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q[i]),
-                                        __builtin_bit_cast(bf16x2, k[i]), a, false);
+    a = __builtin_amdgcn_fdot2_f32_bf16(as_bf16x2(q[i]), as_bf16x2(k[i]), a, false);
   return a;
 }
 template <>
@@ -54,8 +53,7 @@ __device__ __forceinline__ float dot16<F16>(const u32x4 &q, const u32x4 &k) {
   float a = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
-    a = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, q[i]), __builtin_bit_cast(f16x2, k[i]),
-                               a, false);
+    a = __builtin_amdgcn_fdot2(as_f16x2(q[i]), as_f16x2(k[i]), a, false);
   return a;
 }
 

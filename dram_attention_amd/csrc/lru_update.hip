@@ -12,7 +12,7 @@
 // M <= K - T victims consumed; a victim's old page is resident and untouched,
 // hence not among the requests, so no later request observes the eviction.
 // So the kernel does: touch hits and mark first occurrences of missed pages
-// (atomicMax of a position marker in the page->slot map), rank those
+// (atomicMin of a position marker in the page->slot map), rank those
 // occurrences with a block scan, select the M least-recent slots in order
 // (select_sorted), and rewrite both maps in parallel.
 // K > N_hbm (victims may wrap onto pages touched in the same step) keeps the
@@ -51,10 +51,13 @@ struct LeastRecentKey {
   }
 };
 
-__device__ __forceinline__ void atomic_max_signed(int32_t *p, int32_t v) { atomicMax(p, v); }
-__device__ __forceinline__ void atomic_max_signed(int64_t *p, int64_t v) {
-  atomicMax((long long *)p, (long long)v);
+__device__ __forceinline__ void atomic_min_signed(int32_t *p, int32_t v) { atomicMin(p, v); }
+__device__ __forceinline__ void atomic_min_signed(int64_t *p, int64_t v) {
+  atomicMin((long long *)p, (long long)v);
 }
+// Marker a missing page's map entry carries between phases A and B: the
+// position of its first request, shifted far below the "absent" value -1.
+constexpr int64_t kMarkerBase = -(int64_t(1) << 30);
 
 template <typename IdxT, typename MapT, typename TimeT>
 __global__ void __launch_bounds__(kSelThreads)
@@ -104,7 +107,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
           const int32_t v = (int32_t)sel_index(sm.sel.sel[ep]);
           time[v] = now;
           const int64_t old = (int64_t)h2d[v];
-          if (old >= 0) d2h[old] = (MapT)-1;
+          if (old >= 0 && old < n_dram_pages) d2h[old] = (MapT)-1;
           h2d[v] = (MapT)p;
           d2h[p] = (MapT)v;
           mpage[m] = (int32_t)p;
@@ -134,7 +137,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       if (s >= 0)
         time[s] = now;
       else
-        atomic_max_signed(&d2h[p], (MapT)(-(int64_t)k - 2));  // smallest k wins
+        atomic_min_signed(&d2h[p], (MapT)(kMarkerBase + k));  // smallest k wins
     }
     if (t == 0) sm.n_miss = 0;
     __syncthreads();
@@ -145,7 +148,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       int64_t p = -1;
       if (k < K) {
         p = (int64_t)idx[k];
-        if (p >= 0 && p < n_dram_pages) first = (int64_t)d2h[p] == -(int64_t)k - 2;
+        if (p >= 0 && p < n_dram_pages) first = (int64_t)d2h[p] == kMarkerBase + k;
         if (hit) hit[k] = (p >= 0 && p < n_dram_pages && !first) ? 1 : 0;
       }
       const uint64_t m_first = __ballot(first);
@@ -175,7 +178,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       const int32_t p = sm.miss_page[i];
       const int32_t v = (int32_t)sel_index(sm.sel.sel[i]);
       const int64_t old = (int64_t)h2d[v];
-      if (old >= 0) d2h[old] = (MapT)-1;
+      if (old >= 0 && old < n_dram_pages) d2h[old] = (MapT)-1;
       h2d[v] = (MapT)p;
       d2h[p] = (MapT)v;
       time[v] = now;

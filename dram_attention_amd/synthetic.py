@@ -7,8 +7,9 @@ so a CPU checker and the GPU path see bit-identical inputs.
   V ~ N(0,1)
   q_0 ~ N(0,1);  q_t = 0.9 q_{t-1} + 0.44 N(0,1)                  [drift => page reuse]
   planted pages (configs "cpu" and "1m"): every token of the page has
-  key = 3 * q_dir + N(0, 0.3), q_dir = the owning kv group's mean initial
-  query rescaled to norm sqrt(D); they sit outside the initially resident tail.
+  key = 3 * q_dir + N(0, 0.3), q_dir = the initial query of one member of the
+  owning kv group rescaled to norm sqrt(D) (page j: kv head j % Hkv, member
+  (j // Hkv) % rep); they sit outside the initially resident tail.
 Config "cpu" draws K without the channel scale (plain N(0,1)).
 """
 
@@ -98,14 +99,15 @@ def make_prompt(w: Workload, seed: int = 0) -> Prompt:
     planted = []
     if w.planted_pages:
         free = w.n_dram_pages - w.n_hbm_pages  # pages not resident at start
-        group = q0.view(H, w.rep, D).mean(dim=1)
-        q_dir = group / group.norm(dim=-1, keepdim=True) * math.sqrt(D)
+        members = q0.view(H, w.rep, D)
         for j in range(w.planted_pages):
             h = j % H
+            q_dir = members[h, (j // H) % w.rep]
+            q_dir = q_dir / q_dir.norm() * math.sqrt(D)
             page = (j + 1) * free // (w.planted_pages + 1)
             t0 = page * w.page_size
             noise = 0.3 * torch.randn(w.page_size, D, generator=g)
-            k[t0:t0 + w.page_size, h] = 3.0 * q_dir[h] + noise
+            k[t0:t0 + w.page_size, h] = 3.0 * q_dir + noise
             planted.append((h, page))
     return Prompt(k.to(w.dtype)[None], v.to(w.dtype)[None], q0, planted)
 

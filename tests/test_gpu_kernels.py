@@ -9,6 +9,8 @@ import torch
 from oracle import dram_attention_oracle as O
 from tests.golden import lru_kats
 
+from tests.util import close, same
+
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda"
@@ -27,11 +29,11 @@ def test_page_minmax_exact(dtype, H, P, page, D):
 
     k = torch.randn(H, P * page, D, generator=gen(1)).to(dtype)
     got = page_min_max(k.to(DEV), P)
-    assert torch.equal(got.cpu(), O.page_min_max(k, P))
+    assert same(got.cpu(), O.page_min_max(k, P))
     # the layout init_cache hands over: a (S, H, D) tensor viewed as (H, S, D)
     kt = k.transpose(0, 1).contiguous().to(DEV).transpose(0, 1)
     assert not kt.is_contiguous() or H == 1 or P * page == 1
-    assert torch.equal(page_min_max(kt, P).cpu(), O.page_min_max(k, P))
+    assert same(page_min_max(kt, P).cpu(), O.page_min_max(k, P))
 
 
 def test_page_minmax_nan_propagates():
@@ -53,8 +55,8 @@ def test_max_inner_product_reference_cases():
     mm = torch.randn(4, 16, 2, 64, generator=gen(4))
     out = max_inner_product(q.to(DEV), mm.to(DEV))
     assert out.shape == (2, 4, 16) and out.dtype == torch.float32
-    assert torch.allclose(out.cpu(), O.max_ip(q, mm), rtol=1e-3, atol=1e-3)   # :29-38 tolerance
-    assert torch.allclose(out, max_ip_ref(q.to(DEV), mm.to(DEV)), rtol=1e-3, atol=1e-3)
+    assert close(out.cpu(), O.max_ip(q, mm), 1e-3, 1e-3)   # :29-38 tolerance
+    assert close(out, max_ip_ref(q.to(DEV), mm.to(DEV)), 1e-3, 1e-3)
     out16 = max_inner_product(q.half().to(DEV), mm.half().to(DEV))
     assert out16.dtype == torch.float16
     q1, mm1 = torch.randn(1, 1, 1, generator=gen(5)), torch.randn(1, 1, 2, 1, generator=gen(6))
@@ -66,7 +68,7 @@ def test_max_inner_product_reference_cases():
     mmL = torch.randn(32, 1024, 2, 128, generator=gen(8))
     oL = max_inner_product(qL.to(DEV), mmL.to(DEV))
     assert oL.shape == (32, 32, 1024)
-    assert torch.allclose(oL.cpu(), O.max_ip(qL, mmL), rtol=1e-3, atol=1e-3)
+    assert close(oL.cpu(), O.max_ip(qL, mmL), 1e-3, 1e-3)
 
 
 @pytest.mark.parametrize("N,H,D,L", [(4, 8, 128, 515), (8, 2, 64, 130), (1, 3, 128, 4),
@@ -102,7 +104,7 @@ def test_page_score_strided_query_view():
     diff = (out.cpu() - want).abs()
     assert torch.all(diff <= want.abs() * 2.0 ** -7)
     # fp32 output holds bf16-representable values
-    assert torch.equal(out.cpu(), out.cpu().bfloat16().float())
+    assert same(out.cpu(), out.cpu().bfloat16().float())
 
 
 # ------------------------------------------------------------------ top-k
@@ -124,17 +126,17 @@ def test_topk_pages_exact(rows, rep, H, L, k):
     scores = torch.randn(rows, H, L, generator=gen(13))
     got = run_topk(scores, rep, k)
     want = O.select_pages(scores, rows // rep, rep, k)
-    assert torch.equal(got, want)
+    assert same(got, want)
 
 
 @pytest.mark.parametrize("levels", [2, 7, 200])
 def test_topk_pages_ties_lowest_index_first(levels):
     scores = torch.randint(0, levels, (4, 4, 4096), generator=gen(14)).float() - levels / 2
     got = run_topk(scores, 4, 256)
-    assert torch.equal(got, O.select_pages(scores, 1, 4, 256))
+    assert same(got, O.select_pages(scores, 1, 4, 256))
     # bf16-rounded scores, the production case
     s2 = (torch.randn(4, 8, 8192, generator=gen(15)) * 20).bfloat16().float()
-    assert torch.equal(run_topk(s2, 4, 256), O.select_pages(s2, 1, 4, 256))
+    assert same(run_topk(s2, 4, 256), O.select_pages(s2, 1, 4, 256))
 
 
 def test_topk_pages_special_values():
@@ -147,7 +149,7 @@ def test_topk_pages_special_values():
     s[1, 0, 100] = float("nan")           # torch ranks NaN first when descending
     got = run_topk(s, 1, 300)
     want = O.select_pages(s, 2, 1, 300)
-    assert torch.equal(got, want)
+    assert same(got, want)
     assert got[1, 0, 0, 0].item() == 100 and got[1, 0, 0, 1:5].tolist() == [0, 1, 2, 3]
 
 
@@ -159,10 +161,10 @@ def test_topk_for_lru_layout():
     out = torch.empty(H, seq * rep * k, dtype=torch.int64, device=DEV)
     topk_pages(scores.to(DEV), rep, k, out, rep * k, seq * rep * k, k)
     want = O.lru_index_list(O.select_pages(scores, seq, rep, k))
-    assert torch.equal(out.cpu(), want)
+    assert same(out.cpu(), want)
     out32 = torch.empty(H, seq * rep * k, dtype=torch.int32, device=DEV)
     topk_pages(scores.to(DEV), rep, k, out32, rep * k, seq * rep * k, k)
-    assert torch.equal(out32.cpu().long(), want)
+    assert same(out32.cpu().long(), want)
 
 
 # ------------------------------------------------------------------ LRU
@@ -194,7 +196,7 @@ def test_load_lru_cache_reference_kats(name):
     for (h, s), p in case["h2d_after"].items():
         assert h2d[h, s].item() == p
     for h, s, p in case["payload"]:
-        assert torch.equal(hbm[h, s], dram[h, p])
+        assert same(hbm[h, s], dram[h, p])
     assert step.item() == lru_kats.STEP        # the raw function does not advance the step
 
 
@@ -244,7 +246,7 @@ def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat1
                     live[v] = p
                 assert [(p, v) for p, v in got if v >= 0] == \
                     [(p, v) for p, v in miss_o[h] if live[v] == p]
-        assert torch.equal(hbm.cpu(), hbm_o), f"payload, step {s}"
+        assert same(hbm.cpu(), hbm_o), f"payload, step {s}"
 
 
 @pytest.mark.parametrize("H,P,N,K,itype,ttype,pinned", [
@@ -303,17 +305,17 @@ def test_decode_attention_matches_dense(dtype, atol, rtol, Hq, Hkv, D, p_len, c_
     out = decode_attention(q.to(DEV), inter_d[:, :, 0], inter_d[:, :, 1], ckd, cvd, c_len,
                            nk.to(DEV), nv.to(DEV), lse=lse)
     assert out.dtype == dtype
-    assert torch.allclose(out.cpu().float(), want, atol=atol, rtol=rtol)
+    assert close(out.cpu().float(), want, atol, rtol)
     assert torch.allclose(lse.cpu(), want_lse, atol=2e-3 if dtype != torch.float32 else 1e-4)
     # the append happened in place, nothing else moved
-    assert torch.equal(ckd[c_len].cpu(), nk) and torch.equal(cvd[c_len].cpu(), nv)
-    assert torch.equal(ckd[:c_len].cpu(), ck[:c_len]) and torch.equal(ckd[c_len + 1:].cpu(), ck[c_len + 1:])
+    assert same(ckd[c_len].cpu(), nk) and same(cvd[c_len].cpu(), nv)
+    assert same(ckd[:c_len].cpu(), ck[:c_len]) and same(ckd[c_len + 1:].cpu(), ck[c_len + 1:])
     # device-side length gives the same bits
     ckd2, cvd2 = ck.to(DEV), cv.to(DEV)
     out2 = decode_attention(q.to(DEV), inter_d[:, :, 0], inter_d[:, :, 1], ckd2, cvd2,
                             torch.tensor([c_len], dtype=torch.int32, device=DEV),
                             nk.to(DEV), nv.to(DEV))
-    assert torch.equal(out2, out) and torch.equal(ckd2, ckd)
+    assert same(out2, out) and same(ckd2, ckd)
 
 
 def test_decode_attention_large_logits_and_no_append():
@@ -329,7 +331,7 @@ def test_decode_attention_large_logits_and_no_append():
     out = decode_attention(q.to(DEV), k[:, :400].to(DEV), v[:, :400].to(DEV), ck.to(DEV),
                            cv.to(DEV), 300, None, None)
     want, _ = O.attention_partial(q, k, v)
-    assert torch.allclose(out.cpu().float(), want, atol=2e-2, rtol=1e-2)
+    assert close(out.cpu().float(), want, 2e-2, 1e-2)
 
 
 def test_decode_attention_rejects_overflow_and_bad_dim():

@@ -11,6 +11,8 @@ import torch
 from dram_attention_amd.synthetic import WORKLOADS, DecodeInputs, make_prompt
 from oracle import dram_attention_oracle as O
 
+from tests.util import close, same
+
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
@@ -33,7 +35,7 @@ def test_lru_cache_initialization(sample_cache):
     assert torch.all(c.dram_page_to_hbm_page_mapping[:, -102:] == torch.arange(102, device=DEV))
     assert torch.all(c.dram_page_to_hbm_page_mapping[:, :-102] == -1)
     assert c.dram_kv_cache.is_pinned() and c.dram_kv_cache.shape == (4, 512, 16 * 2 * 64)
-    assert torch.equal(c.hbm_kv_cache.cpu(), c.dram_kv_cache[:, -102:])
+    assert same(c.hbm_kv_cache.cpu(), c.dram_kv_cache[:, -102:])
 
 
 def test_lru_cache_load_inline_method(sample_cache):
@@ -46,7 +48,7 @@ def test_lru_cache_load_inline_method(sample_cache):
     assert torch.all(slots >= 0)
     for h in range(4):
         got = sample_cache.hbm_kv_cache[h, slots[h]].cpu()
-        assert torch.equal(got, sample_cache.dram_kv_cache[h, idx[h].cpu()])
+        assert same(got, sample_cache.dram_kv_cache[h, idx[h].cpu()])
 
 
 @pytest.mark.parametrize("page_size", [8, 16, 32])
@@ -84,7 +86,7 @@ def test_lru_cache_get_kv_cache_inline(sample_cache):
     sel = sample_cache.top_k_selector
     scores = sel.scores(query).cpu()
     want = O.select_pages(scores, 10, 1, 10)
-    assert torch.equal(sel.top_k(query, 10).cpu(), want)
+    assert same(sel.top_k(query, 10).cpu(), want)
 
 
 # ------------------------------------------------------------ reference dram_attention_test.py
@@ -126,7 +128,7 @@ def test_module_prefill_then_generate_shapes():
         qs = xq[0, row].float().view(8, 4, 128)
         s = torch.einsum("hrd,thd->hrt", qs, xk[0, : row + 1].float()) / math.sqrt(128)
         want = torch.einsum("hrt,thd->hrd", torch.softmax(s, -1), xv[0, : row + 1].float())
-        assert torch.allclose(out[0, row].float().view(8, 4, 128), want, atol=2e-2, rtol=2e-2)
+        assert close(out[0, row].float().view(8, 4, 128), want, 2e-2, 2e-2)
     q1 = torch.randn(1, 1, 32, 128, device=DEV, dtype=torch.bfloat16, generator=g)
     k1 = torch.randn(1, 1, 8, 128, device=DEV, dtype=torch.bfloat16, generator=g)
     v1 = torch.randn(1, 1, 8, 128, device=DEV, dtype=torch.bfloat16, generator=g)
@@ -154,8 +156,8 @@ def run_parity(w, seed, steps, atol, rtol, device_pos=False):
     assert m.dram_kv_cache_size == o.dram_kv_cache_size == w.dram_tokens
     assert isinstance(m.lru_cache, LRUCache) and o.uses_lru
     lru = m.lru_cache
-    assert torch.equal(lru.top_k_selector.chunk_min_max.cpu(), o.min_max)
-    assert torch.equal(lru.dram_kv_cache, o.dram)
+    assert same(lru.top_k_selector.chunk_min_max.cpu(), o.min_max)
+    assert same(lru.dram_kv_cache, o.dram)
     inputs = DecodeInputs(w, prompt.q0, seed)
     pos = torch.tensor([w.prompt_tokens], dtype=torch.int32, device=DEV)
     hits = total = 0
@@ -169,7 +171,7 @@ def run_parity(w, seed, steps, atol, rtol, device_pos=False):
         own = O.scores_for_selection(xq, o.min_max)
         assert torch.all((scores - own).abs() <= own.abs() * 2.0 ** -7 + 1e-4), f"scores, step {t}"
         want = o.generate(xq, xk, xv, start, scores=scores)
-        assert torch.equal(lru._topk_idx.cpu(), o.last_idx), f"selection, step {t}"
+        assert same(lru._topk_idx.cpu(), o.last_idx), f"selection, step {t}"
         if t == 0:
             for h, page in prompt.planted:
                 assert (o.last_idx[h] == page).any(), "planted page not selected"
@@ -178,13 +180,13 @@ def run_parity(w, seed, steps, atol, rtol, device_pos=False):
         assert np.array_equal(lru.dram_page_to_hbm_page_mapping.cpu().numpy(), o.state.d2h)
         assert np.array_equal(lru.hbm_page_to_dram_page_mapping.cpu().numpy(), o.state.h2d)
         assert np.array_equal(lru._scratch.hit_mask.cpu().numpy().astype(bool), o.last_hit)
-        assert torch.equal(lru.hbm_kv_cache.cpu(), o.hbm), f"slot payload, step {t}"
-        assert torch.allclose(out.cpu().float(), want.float(), atol=atol, rtol=rtol), f"output, step {t}"
+        assert same(lru.hbm_kv_cache.cpu(), o.hbm), f"slot payload, step {t}"
+        assert close(out.cpu().float(), want.float(), atol, rtol), f"output, step {t}"
         hits += int(o.last_hit.sum())
         total += o.last_hit.size
     c = w.prompt_tokens + steps - w.dram_tokens
-    assert torch.equal(m.cache_k[0, :c].cpu(), o.cache_k[:c])
-    assert torch.equal(m.cache_v[0, :c].cpu(), o.cache_v[:c])
+    assert same(m.cache_k[0, :c].cpu(), o.cache_k[:c])
+    assert same(m.cache_v[0, :c].cpu(), o.cache_v[:c])
     return hits / total
 
 
@@ -227,7 +229,7 @@ def test_static_prefix_equals_full_attention():
         ks.append(xk[0]); vs.append(xv[0])
         want, _ = O.attention_partial(xq[0, 0], torch.cat(ks).transpose(0, 1),
                                       torch.cat(vs).transpose(0, 1))
-        assert torch.allclose(out[0, 0].cpu().float(), want, atol=2e-2, rtol=1e-2)
+        assert close(out[0, 0].cpu().float(), want, 2e-2, 1e-2)
 
 
 # ------------------------------------------------------------ full size, by properties
@@ -265,7 +267,7 @@ def test_headline_size_invariants():
         last, last_idx = s_sel[..., -1], sel[..., -1]
         assert torch.all((best_rest < last) | ((best_rest == last) & (best_idx > last_idx)))
         # LRU maps: inverse of each other, all requests resident and touched now
-        assert torch.equal(torch.gather(d2h, 1, h2d), ar.expand(8, N))
+        assert same(torch.gather(d2h, 1, h2d), ar.expand(8, N))
         assert (d2h >= 0).sum().item() == 8 * N
         slots = torch.gather(d2h, 1, idx)
         assert torch.all(slots >= 0)
@@ -273,7 +275,7 @@ def test_headline_size_invariants():
         assert lru.current_step.item() == t + 1
         # payload: every slot holds exactly the page the map names
         want_pages = torch.gather(dram_dev, 1, h2d[:, :, None].expand(-1, -1, dram_dev.shape[2]))
-        assert torch.equal(lru.hbm_kv_cache, want_pages)
+        assert same(lru.hbm_kv_cache, want_pages)
         # attention over all resident slots ++ local window ++ new token
         c = w.prompt_tokens + t - w.dram_tokens
         kk = torch.cat([lru.hbm_kv_cache.view(8, N * 16, 2, 128)[:, :, 0],
@@ -282,5 +284,5 @@ def test_headline_size_invariants():
                         m.cache_v[0, : c + 1].transpose(0, 1)], 1).float()
         s = torch.einsum("hrd,htd->hrt", xq[0, 0].float().view(8, 4, 128), kk) / math.sqrt(128)
         want = torch.einsum("hrt,htd->hrd", torch.softmax(s, -1), vv).reshape(32, 128)
-        assert torch.allclose(out[0, 0].float(), want, atol=2e-2, rtol=1e-2)
-        assert torch.equal(m.cache_k[0, c], xk[0, 0]) and torch.equal(m.cache_v[0, c], xv[0, 0])
+        assert close(out[0, 0].float(), want, 2e-2, 1e-2)
+        assert same(m.cache_k[0, c], xk[0, 0]) and same(m.cache_v[0, c], xv[0, 0])

@@ -114,6 +114,16 @@ def test_synthetic_workloads():
                                           c.pages_per_q_head))
     for h, page in p1.planted:
         assert (idx[h] == page).any()
+    # ... also with outlier channels and 8 queries per kv head (the 1M layer shape, scaled)
+    w8 = w5.scaled(dram_tokens=8192, local_cache=512, lru_tokens=2048, top_k_tokens=256,
+                   planted_pages=8)
+    p8 = make_prompt(w8, 2)
+    xq8, _, _ = DecodeInputs(w8, p8.q0, 2).next()
+    mm8 = O.page_min_max(p8.k[0, : w8.dram_tokens].transpose(0, 1), w8.n_dram_pages)
+    idx8 = O.lru_index_list(O.select_pages(O.scores_for_selection(xq8, mm8), 1, w8.rep,
+                                           w8.pages_per_q_head))
+    for h, page in p8.planted:
+        assert (idx8[h] == page).any()
     a, b = DecodeInputs(c, p1.q0, 0), DecodeInputs(c, p1.q0, 0)
     for _ in range(3):
         for x, y in zip(a.next(), b.next()):
