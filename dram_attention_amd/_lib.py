@@ -47,7 +47,7 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_int, c_int, c_int, c_int64, c_int, c_void_p, c_int, c_void_p,
          c_int64, c_int, c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p,
-         c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+         c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     ),
     "da_pages_gather": (
         c_int,
@@ -55,14 +55,36 @@ SIGNATURES = {
          c_void_p, c_int, c_int, c_void_p],
     ),
     "da_decode_attention_workspace_bytes": (
-        c_size_t, [c_int, c_int, c_int, c_int, c_int64, c_int64]),
+        c_size_t, [c_int, c_int, c_int, c_int, c_int64, c_int64, c_int64]),
     "da_decode_attention": (
         c_int,
         [c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_int64,
          c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
          c_void_p, c_int64, c_float, c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p],
     ),
+    "da_decode_attention_paged": (
+        c_int,
+        [c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_int64,
+         c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+         c_void_p, c_int64, c_float, c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p,
+         c_void_p],
+    ),
 }
+
+
+class PagedOverlap(ctypes.Structure):
+    """struct da_paged_overlap of the header."""
+
+    _fields_ = [
+        ("page_size", ctypes.c_int32),
+        ("phase", ctypes.c_int32),
+        ("slot_epoch", c_void_p),
+        ("slot_epoch_head_stride", c_int64),
+        ("epoch", c_void_p),
+        ("miss_slot", c_void_p),
+        ("miss_count", c_void_p),
+        ("miss_capacity", ctypes.c_int32),
+    ]
 
 _lib = None
 

@@ -16,6 +16,14 @@
 // registers.  States are merged by shuffles inside the wave, through LDS
 // across the four waves, and written as one fp32 partial per (chunk, q head);
 // a second kernel merges the partials of all chunks.
+//
+// Paged prefix with overlap: when the prefix is the slot array of an LRU page
+// cache whose missed pages are still being streamed in on another stream, the
+// work is issued in two phases.  Phase 1 covers the local segment and every
+// slot that was NOT re-assigned in this step (slot_epoch != current epoch);
+// phase 2, issued once the page stream has finished, covers the re-assigned
+// slots through the miss list and then merges everything.  Both phases are the
+// same kernel; a chunk id says which segment a block works on.
 #include "common.hpp"
 
 namespace da {
@@ -36,8 +44,7 @@ template <>
 __device__ __forceinline__ float dot16<F32>(const u32x4 &q, const u32x4 &k) {
   float a = 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
-    a = fmaf(as_f32(q[i]), as_f32(k[i]), a);
+  for (int i = 0; i < 4; ++i) a = fmaf(as_f32(q[i]), as_f32(k[i]), a);
   return a;
 }
 template <>
@@ -52,8 +59,7 @@ template <>
 __device__ __forceinline__ float dot16<F16>(const u32x4 &q, const u32x4 &k) {
   float a = 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
-    a = __builtin_amdgcn_fdot2(as_f16x2(q[i]), as_f16x2(k[i]), a, false);
+  for (int i = 0; i < 4; ++i) a = __builtin_amdgcn_fdot2(as_f16x2(q[i]), as_f16x2(k[i]), a, false);
   return a;
 }
 
@@ -70,12 +76,34 @@ struct AttnArgs {
   int64_t new_head_stride;
   float scale_log2;  // softmax scale * log2(e)
   int chunk;         // tokens per block
-  int n_pchunks;     // chunks of the prefix segment (the rest belong to the local segment)
-  int n_chunks;      // grid.x
+  // chunk ids: [0, n_pchunks) prefix, [n_pchunks, +n_lchunks) local, then n_tchunks tail
+  int n_pchunks, n_lchunks, n_tchunks;
+  int chunk_base;  // chunk id of blockIdx.x == 0 in this launch
   int n_q_heads;
-  float *part_ml;   // (n_chunks, Hq, 2): running max (log2 domain), sum
-  float *part_acc;  // (n_chunks, Hq, D)
+  float *part_ml;   // (chunks, Hq, 2): running max (log2 domain), sum
+  float *part_acc;  // (chunks, Hq, D)
+  // paged prefix with overlap (all null / 0 otherwise)
+  int page_size;
+  const int32_t *slot_epoch;  // (Hkv, p_len / page_size): epoch of a slot's last re-assignment
+  int64_t slot_epoch_head_stride;
+  const int32_t *epoch;       // the current epoch (one int32)
+  const int32_t *miss_slot;   // (Hkv, miss_capacity) slots re-assigned in this epoch
+  const int32_t *miss_count;  // (Hkv)
+  int miss_capacity;
 };
+
+struct LocalLen {
+  int64_t c_len;  // rows already in the local cache (clamped to its capacity)
+  bool has_new;   // the new token is appended and attended
+};
+__device__ __forceinline__ LocalLen local_len(const AttnArgs &a) {
+  int64_t c_len = a.c_len;
+  if (a.c_len_dev) c_len = *a.c_len_dev;
+  if (c_len < 0) c_len = 0;
+  const bool has_new = a.new_k != nullptr && c_len < a.c_capacity;
+  if (c_len > a.c_capacity) c_len = a.c_capacity;
+  return {c_len, has_new};
+}
 
 template <typename T, int kLanes, int kRows>
 __global__ void __launch_bounds__(kAttnThreads)
@@ -90,23 +118,29 @@ decode_attention_split_kernel(const AttnArgs a) {
   const int g = lane / kLanes;
   const int h = blockIdx.y;
   const int row0 = blockIdx.z * kRows;  // first query row of the GQA group handled here
-  const int chunk_id = blockIdx.x;
+  const int chunk_id = a.chunk_base + blockIdx.x;
 
   // Which segment, which token range.
-  const bool local = chunk_id >= a.n_pchunks;
-  int64_t c_len = a.c_len;
-  if (a.c_len_dev) c_len = *a.c_len_dev;
-  if (c_len < 0) c_len = 0;
-  const bool has_new = a.new_k != nullptr && c_len < a.c_capacity;
-  if (c_len > a.c_capacity) c_len = a.c_capacity;
-  const int64_t seg_len = local ? c_len + (has_new ? 1 : 0) : a.p_len;
-  const int64_t t_begin = (int64_t)(local ? chunk_id - a.n_pchunks : chunk_id) * a.chunk;
+  const int kind = chunk_id < a.n_pchunks ? 0 : (chunk_id < a.n_pchunks + a.n_lchunks ? 1 : 2);
+  const LocalLen ll = local_len(a);
+  const int64_t c_len = ll.c_len;
+  int64_t seg_len, t_begin;
+  if (kind == 0) {
+    seg_len = a.p_len;
+    t_begin = (int64_t)chunk_id * a.chunk;
+  } else if (kind == 1) {
+    seg_len = c_len + (ll.has_new ? 1 : 0);
+    t_begin = (int64_t)(chunk_id - a.n_pchunks) * a.chunk;
+  } else {
+    seg_len = (int64_t)a.miss_count[h] * a.page_size;
+    t_begin = (int64_t)(chunk_id - a.n_pchunks - a.n_lchunks) * a.chunk;
+  }
   if (t_begin >= seg_len) return;  // the merge kernel skips this chunk as well
   const int64_t t_end = t_begin + a.chunk < seg_len ? t_begin + a.chunk : seg_len;
 
   const char *kbase, *vbase;
   int64_t tok_stride_b;
-  if (local) {
+  if (kind == 1) {
     kbase = a.ck + h * a.c_head_stride * T::kBytes + c * 16;
     vbase = a.cv + h * a.c_head_stride * T::kBytes + c * 16;
     tok_stride_b = a.c_tok_stride * T::kBytes;
@@ -116,10 +150,14 @@ decode_attention_split_kernel(const AttnArgs a) {
     tok_stride_b = a.p_tok_stride * T::kBytes;
   }
   const char *newk = nullptr, *newv = nullptr;
-  if (local && has_new) {
+  if (kind == 1 && ll.has_new) {
     newk = a.new_k + h * a.new_head_stride * T::kBytes + c * 16;
     newv = a.new_v + h * a.new_head_stride * T::kBytes + c * 16;
   }
+  const bool skip_fresh = kind == 0 && a.slot_epoch != nullptr;
+  const int32_t epoch_now = skip_fresh ? *a.epoch : 0;
+  const int32_t *slot_epoch = skip_fresh ? a.slot_epoch + h * a.slot_epoch_head_stride : nullptr;
+  const int32_t *miss_slot = kind == 2 ? a.miss_slot + (int64_t)h * a.miss_capacity : nullptr;
 
   u32x4 qv[kRows];
 #pragma unroll
@@ -148,12 +186,26 @@ decode_attention_split_kernel(const AttnArgs a) {
     for (int u = 0; u < kAttnUnroll; ++u) {
       const int64_t tok = t0 + (int64_t)u * kStepTokens;
       valid[u] = tok < t_end;
-      const int64_t tk = valid[u] ? tok : t_begin;  // clamp the address, mask the score
+      int64_t tk = valid[u] ? tok : t_begin;  // clamp the address, mask the score
+      if (skip_fresh) {
+        // a slot that is being rewritten right now is left to the tail pass
+        if (slot_epoch[tk / a.page_size] == epoch_now) valid[u] = false;
+      } else if (kind == 2) {
+        const int32_t slot = miss_slot[tk / a.page_size];
+        if (slot < 0) valid[u] = false;  // entry superseded later in the same step
+        tk = (int64_t)(slot < 0 ? 0 : slot) * a.page_size + tk % a.page_size;
+      }
       const bool is_new = newk != nullptr && tk == c_len;
       const char *kp = is_new ? newk : kbase + tk * tok_stride_b;
       const char *vp = is_new ? newv : vbase + tk * tok_stride_b;
-      kk[u] = load16(kp);
-      vv[u] = load16(vp);
+      if (skip_fresh && !valid[u]) {
+        // never touch memory another stream is writing: torn values could be NaN
+        kk[u] = u32x4{0, 0, 0, 0};
+        vv[u] = u32x4{0, 0, 0, 0};
+      } else {
+        kk[u] = load16(kp);
+        vv[u] = load16(vp);
+      }
       if (is_new && valid[u] && blockIdx.z == 0) {
         // the append: this lane group owns the new token's row
         store16(a.ck + (h * a.c_head_stride + c_len * a.c_tok_stride) * T::kBytes + c * 16, kk[u]);
@@ -251,65 +303,57 @@ decode_attention_split_kernel(const AttnArgs a) {
   }
 }
 
-// Merge the partials of one query head.  One 256-thread block per head; a
-// thread owns four adjacent output channels of every (256 / (D/4))-th chunk,
-// so the chunk rows are read as 16-byte lanes and the chunk loop is short.
+// Merge the partials of one query head.  One 512-thread block per head.  The
+// softmax statistics are tiny, so every wave reduces them for itself (no
+// barrier); then a thread owns four adjacent output channels of every 16th
+// (at D = 128) chunk, reads the partial rows as 16-byte lanes, and the chunk
+// lanes are folded through LDS.
+constexpr int kMergeThreads = 512;
+
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kMergeThreads)
 decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__ out,
                               int64_t out_head_stride, float *__restrict__ lse_out) {
   const int hq = blockIdx.x;
   const int t = threadIdx.x;
-  int64_t c_len = a.c_len;
-  if (a.c_len_dev) c_len = *a.c_len_dev;
-  if (c_len < 0) c_len = 0;
-  const bool has_new = a.new_k != nullptr && c_len < a.c_capacity;
-  if (c_len > a.c_capacity) c_len = a.c_capacity;
-  const int64_t l_len = c_len + (has_new ? 1 : 0);
-  const int n_p = (int)((a.p_len + a.chunk - 1) / a.chunk);  // live prefix chunks
-  const int n_l = (int)((l_len + a.chunk - 1) / a.chunk);    // live local chunks
-  const int n_live = n_p + n_l;
+  const int lane = t & 63;
+  const LocalLen ll = local_len(a);
+  const int64_t l_len = ll.c_len + (ll.has_new ? 1 : 0);
+  const int n_p = a.n_pchunks;                              // live prefix chunks (all of them)
+  const int n_l = (int)((l_len + a.chunk - 1) / a.chunk);   // live local chunks
+  int n_t = 0;                                              // live tail chunks
+  if (a.n_tchunks > 0) {
+    const int64_t tail = (int64_t)a.miss_count[hq / a.rep] * a.page_size;
+    n_t = (int)((tail + a.chunk - 1) / a.chunk);
+  }
+  const int n_live = n_p + n_l + n_t;
+  // i-th live chunk -> chunk id
+  auto chunk_of = [&](int i) {
+    return i < n_p + n_l ? i : a.n_pchunks + a.n_lchunks + (i - n_p - n_l);
+  };
 
-  __shared__ float sm_red[256];
-  __shared__ float sm_acc[256 * 4];
-  // pass 1: global max over the live chunks
   float mx = kMinusHuge;
-  for (int i = t; i < n_live; i += 256) {
-    const int ch = i < n_p ? i : a.n_pchunks + (i - n_p);
-    mx = fmaxf(mx, a.part_ml[((int64_t)ch * a.n_q_heads + hq) * 2]);
-  }
-  sm_red[t] = mx;
-  __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) {
-    if (t < s) sm_red[t] = fmaxf(sm_red[t], sm_red[t + s]);
-    __syncthreads();
-  }
-  mx = sm_red[0];
-  __syncthreads();
-  // pass 2: the softmax denominator
+  for (int i = lane; i < n_live; i += 64)
+    mx = fmaxf(mx, a.part_ml[((int64_t)chunk_of(i) * a.n_q_heads + hq) * 2]);
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
   float lt = 0.f;
-  for (int i = t; i < n_live; i += 256) {
-    const int ch = i < n_p ? i : a.n_pchunks + (i - n_p);
-    const float *ml = a.part_ml + ((int64_t)ch * a.n_q_heads + hq) * 2;
+  for (int i = lane; i < n_live; i += 64) {
+    const float *ml = a.part_ml + ((int64_t)chunk_of(i) * a.n_q_heads + hq) * 2;
     lt += ml[1] * fast_exp2(ml[0] - mx);
   }
-  sm_red[t] = lt;
-  __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) {
-    if (t < s) sm_red[t] += sm_red[t + s];
-    __syncthreads();
-  }
-  lt = sm_red[0];
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) lt += __shfl_xor(lt, d, 64);
   const float inv = lt > 0.f ? 1.f / lt : 0.f;
-  // pass 3: weighted sum of the partial output rows
-  const int quads = head_dim / 4;        // 16-byte lanes per row (head_dim % 4 == 0 here)
-  const int lanes_c = 256 / quads;       // chunk lanes
+
+  __shared__ float sm_acc[kMergeThreads * 4];
+  const int quads = head_dim / 4;              // 16-byte lanes per row (head_dim % 4 == 0 here)
+  const int lanes_c = kMergeThreads / quads;   // chunk lanes
   const int qd = t % quads, cl = t / quads;
   float at[4] = {0.f, 0.f, 0.f, 0.f};
   if (cl < lanes_c) {
     for (int i = cl; i < n_live; i += lanes_c) {
-      const int ch = i < n_p ? i : a.n_pchunks + (i - n_p);
-      const int64_t slot = (int64_t)ch * a.n_q_heads + hq;
+      const int64_t slot = (int64_t)chunk_of(i) * a.n_q_heads + hq;
       const float w = fast_exp2(a.part_ml[slot * 2] - mx);
       const float4 v = *(const float4 *)(a.part_acc + slot * head_dim + qd * 4);
       at[0] = fmaf(v.x, w, at[0]);
@@ -321,7 +365,7 @@ decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__
 #pragma unroll
   for (int i = 0; i < 4; ++i) sm_acc[t * 4 + i] = at[i];
   __syncthreads();
-  for (int d = t; d < head_dim; d += 256) {
+  for (int d = t; d < head_dim; d += kMergeThreads) {
     float s = 0.f;
     for (int c2 = 0; c2 < lanes_c; ++c2) s += sm_acc[(c2 * quads + d / 4) * 4 + (d & 3)];
     store_elem<T>(out, (int64_t)hq * out_head_stride + d, s * inv);
@@ -347,81 +391,98 @@ static int lanes_of(int head_dim, int dtype) {
   return (lanes >= 4 && lanes <= 64 && is_pow2(lanes)) ? lanes : 0;
 }
 
+struct ChunkPlan {
+  int chunk, n_p, n_l, n_t;
+  int64_t total() const { return (int64_t)n_p + n_l + n_t; }
+};
+// The chunk geometry of a launch; a function of the shapes only, so that the
+// workspace query and every phase of a step agree on it.
+static ChunkPlan plan_chunks(int n_kv_heads, int lanes, int64_t p_len, int64_t c_capacity,
+                             int64_t miss_tokens) {
+  const int step_tokens = kAttnWaves * (64 / lanes);
+  ChunkPlan p;
+  p.chunk = pick_chunk(p_len + c_capacity, n_kv_heads, step_tokens);
+  p.n_p = (int)ceil_div(p_len, p.chunk);
+  p.n_l = (int)ceil_div(c_capacity, p.chunk);
+  p.n_t = (int)ceil_div(miss_tokens, p.chunk);
+  return p;
+}
+
 static size_t attn_workspace_bytes(int n_q_heads, int head_dim, int64_t n_chunks) {
   return (size_t)n_chunks * n_q_heads * (head_dim + 2) * sizeof(float);
 }
 
-// Upper bound of the chunk count for a geometry (chunk size is fixed by the
-// same rule at launch, from the same numbers).
-static int64_t plan_chunks(int n_q_heads_unused, int n_kv_heads, int lanes, int64_t p_len,
-                           int64_t c_capacity, int *chunk_out, int *n_p_out) {
-  (void)n_q_heads_unused;
-  const int step_tokens = kAttnWaves * (64 / lanes);
-  const int chunk = pick_chunk(p_len + c_capacity, n_kv_heads, step_tokens);
-  const int64_t n_p = ceil_div(p_len, chunk);
-  const int64_t n_l = ceil_div(c_capacity, chunk);
-  if (chunk_out) *chunk_out = chunk;
-  if (n_p_out) *n_p_out = (int)n_p;
-  return n_p + n_l;
-}
-
 template <typename T, int kLanes>
-static void launch_split(const AttnArgs &a, int n_kv_heads, hipStream_t s) {
+static void launch_split(AttnArgs a, int first_chunk, int n_launch, int n_kv_heads,
+                         hipStream_t s) {
+  if (n_launch <= 0) return;
+  a.chunk_base = first_chunk;
   const int rep = a.rep;
   if (rep <= 1) {
-    dim3 grid(a.n_chunks, n_kv_heads, 1);
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 1>), grid, dim3(kAttnThreads), 0,
-                       s, a);
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 1>),
+                       dim3(n_launch, n_kv_heads, 1), dim3(kAttnThreads), 0, s, a);
   } else if (rep == 2) {
-    dim3 grid(a.n_chunks, n_kv_heads, 1);
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 2>), grid, dim3(kAttnThreads), 0,
-                       s, a);
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 2>),
+                       dim3(n_launch, n_kv_heads, 1), dim3(kAttnThreads), 0, s, a);
   } else {
-    dim3 grid(a.n_chunks, n_kv_heads, (unsigned)ceil_div(rep, 4));
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 4>), grid, dim3(kAttnThreads), 0,
-                       s, a);
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 4>),
+                       dim3(n_launch, n_kv_heads, (unsigned)ceil_div(rep, 4)),
+                       dim3(kAttnThreads), 0, s, a);
   }
 }
 
+// phase bit 1: prefix (minus fresh slots) + local segment; bit 2: tail + merge.
 template <typename T>
-static int launch_attention(const AttnArgs &a, int n_kv_heads, int lanes, int head_dim, void *out,
-                            int64_t out_head_stride, float *lse_out, hipStream_t s) {
-  switch (lanes) {
-    case 4: launch_split<T, 4>(a, n_kv_heads, s); break;
-    case 8: launch_split<T, 8>(a, n_kv_heads, s); break;
-    case 16: launch_split<T, 16>(a, n_kv_heads, s); break;
-    case 32: launch_split<T, 32>(a, n_kv_heads, s); break;
-    case 64: launch_split<T, 64>(a, n_kv_heads, s); break;
+static int launch_attention(const AttnArgs &a, int phase, int n_kv_heads, int lanes, int head_dim,
+                            void *out, int64_t out_head_stride, float *lse_out, hipStream_t s) {
+#define DA_ATTN_LAUNCH(first, count)                                  \
+  switch (lanes) {                                                    \
+    case 4: launch_split<T, 4>(a, first, count, n_kv_heads, s); break;   \
+    case 8: launch_split<T, 8>(a, first, count, n_kv_heads, s); break;   \
+    case 16: launch_split<T, 16>(a, first, count, n_kv_heads, s); break; \
+    case 32: launch_split<T, 32>(a, first, count, n_kv_heads, s); break; \
+    case 64: launch_split<T, 64>(a, first, count, n_kv_heads, s); break; \
   }
-  int rc = launch_status("da_decode_attention(split)");
-  if (rc) return rc;
-  hipLaunchKernelGGL(decode_attention_merge_kernel<T>, dim3(a.n_q_heads), dim3(256), 0, s, a,
-                     head_dim, (char *)out, out_head_stride, lse_out);
-  return launch_status("da_decode_attention(merge)");
+  if (phase & 1) {
+    DA_ATTN_LAUNCH(0, a.n_pchunks + a.n_lchunks)
+    int rc = launch_status("da_decode_attention(split)");
+    if (rc) return rc;
+  }
+  if (phase & 2) {
+    if (a.n_tchunks > 0) {
+      DA_ATTN_LAUNCH(a.n_pchunks + a.n_lchunks, a.n_tchunks)
+      int rc = launch_status("da_decode_attention(tail)");
+      if (rc) return rc;
+    }
+    hipLaunchKernelGGL(decode_attention_merge_kernel<T>, dim3(a.n_q_heads), dim3(kMergeThreads), 0,
+                       s, a, head_dim, (char *)out, out_head_stride, lse_out);
+    return launch_status("da_decode_attention(merge)");
+  }
+#undef DA_ATTN_LAUNCH
+  return DA_OK;
 }
 
 }  // namespace da
 
 extern "C" size_t da_decode_attention_workspace_bytes(int n_q_heads, int n_kv_heads,
                                                       int head_dim, int dtype, int64_t p_len,
-                                                      int64_t c_capacity) {
+                                                      int64_t c_capacity, int64_t miss_tokens) {
   using namespace da;
-  if (n_q_heads <= 0 || n_kv_heads <= 0 || p_len < 0 || c_capacity < 0) return 0;
+  if (n_q_heads <= 0 || n_kv_heads <= 0 || p_len < 0 || c_capacity < 0 || miss_tokens < 0)
+    return 0;
   const int lanes = lanes_of(head_dim, dtype);
   if (!lanes) return 0;
-  const int64_t n = plan_chunks(n_q_heads, n_kv_heads, lanes, p_len, c_capacity, nullptr, nullptr);
-  return attn_workspace_bytes(n_q_heads, head_dim, n) + 16;
+  const ChunkPlan p = plan_chunks(n_kv_heads, lanes, p_len, c_capacity, miss_tokens);
+  return attn_workspace_bytes(n_q_heads, head_dim, p.total()) + 16;
 }
 
-extern "C" int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
-                                   int n_kv_heads, int head_dim, int dtype, const void *pk,
-                                   const void *pv, int64_t p_tok_stride, int64_t p_head_stride,
-                                   int64_t p_len, void *ck, void *cv, int64_t c_tok_stride,
-                                   int64_t c_head_stride, int64_t c_capacity, int64_t c_len,
-                                   const int32_t *c_len_dev, const void *new_k,
-                                   const void *new_v, int64_t new_head_stride, float scale,
-                                   void *out, int64_t out_head_stride, float *lse_out,
-                                   void *workspace, size_t workspace_bytes, void *stream) {
+extern "C" int da_decode_attention_paged(
+    const void *q, int64_t q_head_stride, int n_q_heads, int n_kv_heads, int head_dim, int dtype,
+    const void *pk, const void *pv, int64_t p_tok_stride, int64_t p_head_stride, int64_t p_len,
+    void *ck, void *cv, int64_t c_tok_stride, int64_t c_head_stride, int64_t c_capacity,
+    int64_t c_len, const int32_t *c_len_dev, const void *new_k, const void *new_v,
+    int64_t new_head_stride, float scale, void *out, int64_t out_head_stride, float *lse_out,
+    void *workspace, size_t workspace_bytes, const da_paged_overlap *overlap, void *stream) {
   using namespace da;
   DA_REQUIRE(n_q_heads > 0 && n_kv_heads > 0 && n_q_heads % n_kv_heads == 0,
              "da_decode_attention: %d query heads do not split over %d kv heads", n_q_heads,
@@ -455,7 +516,7 @@ extern "C" int da_decode_attention(const void *q, int64_t q_head_stride, int n_q
              "da_decode_attention: rows must be 16-byte aligned");
   if (n_kv_heads > 65535) return fail(DA_ENOTSUP, "da_decode_attention: too many kv heads");
 
-  AttnArgs a;
+  AttnArgs a = {};
   a.q = (const char *)q;
   a.q_head_stride = q_head_stride;
   a.rep = n_q_heads / n_kv_heads;
@@ -476,32 +537,65 @@ extern "C" int da_decode_attention(const void *q, int64_t q_head_stride, int n_q
   a.new_head_stride = new_head_stride;
   a.scale_log2 = scale * kLog2e;
   a.n_q_heads = n_q_heads;
-  int chunk = 0, n_p = 0;
-  const int64_t n_chunks = plan_chunks(n_q_heads, n_kv_heads, lanes, p_len, c_capacity, &chunk, &n_p);
-  a.chunk = chunk;
-  a.n_pchunks = n_p;
-  a.n_chunks = (int)n_chunks;
-  const size_t need = attn_workspace_bytes(n_q_heads, head_dim, n_chunks);
+  int phase = 3;
+  int64_t miss_tokens = 0;
+  if (overlap) {
+    DA_REQUIRE(overlap->page_size > 0 && p_len % overlap->page_size == 0,
+               "da_decode_attention: the paged prefix must be whole pages");
+    DA_REQUIRE(overlap->slot_epoch && overlap->epoch && overlap->miss_slot &&
+                   overlap->miss_count && overlap->miss_capacity >= 0,
+               "da_decode_attention: incomplete overlap description");
+    DA_REQUIRE(overlap->phase >= 1 && overlap->phase <= 3, "da_decode_attention: bad phase %d",
+               overlap->phase);
+    a.page_size = overlap->page_size;
+    a.slot_epoch = overlap->slot_epoch;
+    a.slot_epoch_head_stride = overlap->slot_epoch_head_stride;
+    a.epoch = overlap->epoch;
+    a.miss_slot = overlap->miss_slot;
+    a.miss_count = overlap->miss_count;
+    a.miss_capacity = overlap->miss_capacity;
+    miss_tokens = (int64_t)overlap->miss_capacity * overlap->page_size;
+    phase = overlap->phase;
+  }
+  const ChunkPlan p = plan_chunks(n_kv_heads, lanes, p_len, c_capacity, miss_tokens);
+  a.chunk = p.chunk;
+  a.n_pchunks = p.n_p;
+  a.n_lchunks = p.n_l;
+  a.n_tchunks = p.n_t;
+  const size_t need = attn_workspace_bytes(n_q_heads, head_dim, p.total());
   DA_REQUIRE(workspace_bytes >= need, "da_decode_attention: workspace %zu < %zu bytes",
              workspace_bytes, need);
-  DA_REQUIRE((uintptr_t)workspace % 16 == 0, "da_decode_attention: workspace must be 16-byte aligned");
+  DA_REQUIRE((uintptr_t)workspace % 16 == 0,
+             "da_decode_attention: workspace must be 16-byte aligned");
   a.part_acc = (float *)workspace;
-  a.part_ml = a.part_acc + (size_t)n_chunks * n_q_heads * head_dim;
+  a.part_ml = a.part_acc + (size_t)p.total() * n_q_heads * head_dim;
   hipStream_t s = (hipStream_t)stream;
-  if (n_chunks == 0) {
-    // nothing to attend over: the merge kernel alone writes zeros / -inf
-    a.n_chunks = 0;
-  }
+  if (p.n_p + p.n_l == 0) return fail(DA_EINVAL, "da_decode_attention: no key/value rows at all");
   switch (dtype) {
     case DA_F32:
-      if (n_chunks == 0) break;
-      return launch_attention<F32>(a, n_kv_heads, lanes, head_dim, out, out_head_stride, lse_out, s);
+      return launch_attention<F32>(a, phase, n_kv_heads, lanes, head_dim, out, out_head_stride,
+                                   lse_out, s);
     case DA_F16:
-      if (n_chunks == 0) break;
-      return launch_attention<F16>(a, n_kv_heads, lanes, head_dim, out, out_head_stride, lse_out, s);
+      return launch_attention<F16>(a, phase, n_kv_heads, lanes, head_dim, out, out_head_stride,
+                                   lse_out, s);
     default:
-      if (n_chunks == 0) break;
-      return launch_attention<BF16>(a, n_kv_heads, lanes, head_dim, out, out_head_stride, lse_out, s);
+      return launch_attention<BF16>(a, phase, n_kv_heads, lanes, head_dim, out, out_head_stride,
+                                    lse_out, s);
   }
-  return fail(DA_EINVAL, "da_decode_attention: no key/value rows at all");
+}
+
+extern "C" int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
+                                   int n_kv_heads, int head_dim, int dtype, const void *pk,
+                                   const void *pv, int64_t p_tok_stride, int64_t p_head_stride,
+                                   int64_t p_len, void *ck, void *cv, int64_t c_tok_stride,
+                                   int64_t c_head_stride, int64_t c_capacity, int64_t c_len,
+                                   const int32_t *c_len_dev, const void *new_k,
+                                   const void *new_v, int64_t new_head_stride, float scale,
+                                   void *out, int64_t out_head_stride, float *lse_out,
+                                   void *workspace, size_t workspace_bytes, void *stream) {
+  return da_decode_attention_paged(q, q_head_stride, n_q_heads, n_kv_heads, head_dim, dtype, pk,
+                                   pv, p_tok_stride, p_head_stride, p_len, ck, cv, c_tok_stride,
+                                   c_head_stride, c_capacity, c_len, c_len_dev, new_k, new_v,
+                                   new_head_stride, scale, out, out_head_stride, lse_out,
+                                   workspace, workspace_bytes, nullptr, stream);
 }

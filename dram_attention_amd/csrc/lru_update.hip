@@ -49,6 +49,17 @@ struct LeastRecentKey {
   __device__ __forceinline__ uint32_t operator()(int i) const {
     return ~time_order_key<TimeT>(time[i]);
   }
+  __device__ __forceinline__ void load4(int i, uint32_t *k) const {
+    TimeT v[4];
+    if (((uintptr_t)time & 15) == 0) {
+      *(u32x4 *)v = *(const u32x4 *)(time + i);
+    } else {
+#pragma unroll
+      for (int x = 0; x < 4; ++x) v[x] = time[i + x];
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x) k[x] = ~time_order_key<TimeT>(v[x]);
+  }
 };
 
 __device__ __forceinline__ void atomic_min_signed(int32_t *p, int32_t v) { atomicMin(p, v); }
@@ -66,7 +77,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
                   TimeT *time_all, int64_t time_head_stride, MapT *d2h_all,
                   int64_t d2h_head_stride, MapT *h2d_all, int64_t h2d_head_stride,
                   uint8_t *hit_mask, int32_t *miss_page_out, int32_t *miss_slot_out,
-                  int32_t *miss_count, int32_t *ticket, int serial) {
+                  int32_t *miss_count, int32_t *slot_epoch_all, int32_t *ticket, int serial) {
   __shared__ LruShared sm;
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -79,6 +90,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
   uint8_t *hit = hit_mask ? hit_mask + (int64_t)h * K : nullptr;
   int32_t *mpage = miss_page_out + (int64_t)h * K;
   int32_t *mslot = miss_slot_out + (int64_t)h * K;
+  int32_t *slot_epoch = slot_epoch_all ? slot_epoch_all + (int64_t)h * n_hbm : nullptr;
 
   const int32_t step = *step_ptr + (bump ? 1 : 0);
   const TimeT now = (TimeT)step;
@@ -93,7 +105,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
     }
     __syncthreads();
     LeastRecentKey<TimeT> key{time};
-    select_sorted(key, n_hbm, n_hbm, sm.sel);  // full stable order of the slots
+    const uint32_t *order = select_sorted(key, n_hbm, n_hbm, sm.sel);  // full stable order
     if (t == 0) {
       int ep = 0, m = 0;
       for (int k = 0; k < K; ++k) {
@@ -104,7 +116,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
         }
         const int64_t s = (int64_t)d2h[p];
         if (s < 0) {
-          const int32_t v = (int32_t)sel_index(sm.sel.sel[ep]);
+          const int32_t v = (int32_t)order[ep];
           time[v] = now;
           const int64_t old = (int64_t)h2d[v];
           if (old >= 0 && old < n_dram_pages) d2h[old] = (MapT)-1;
@@ -112,6 +124,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
           d2h[p] = (MapT)v;
           mpage[m] = (int32_t)p;
           mslot[m] = v;
+          if (slot_epoch) slot_epoch[v] = step;
           ++m;
           ep = ep + 1 == n_hbm ? 0 : ep + 1;
           if (hit) hit[k] = 0;
@@ -169,14 +182,15 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
     }
     const int m = (int)sm.n_miss;
     // -- phase C: the m least recently used slots, in eviction order ---------
+    const uint32_t *victims = nullptr;
     if (m > 0) {
       LeastRecentKey<TimeT> key{time};
-      select_sorted(key, n_hbm, m, sm.sel);
+      victims = select_sorted(key, n_hbm, m, sm.sel);
     }
     // -- phase D: hand slot i to the i-th distinct missed page ---------------
     for (int i = t; i < m; i += kSelThreads) {
       const int32_t p = sm.miss_page[i];
-      const int32_t v = (int32_t)sel_index(sm.sel.sel[i]);
+      const int32_t v = (int32_t)victims[i];
       const int64_t old = (int64_t)h2d[v];
       if (old >= 0 && old < n_dram_pages) d2h[old] = (MapT)-1;
       h2d[v] = (MapT)p;
@@ -184,6 +198,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       time[v] = now;
       mpage[i] = p;
       mslot[i] = v;
+      if (slot_epoch) slot_epoch[v] = step;
     }
     if (t == 0) miss_count[h] = m;
   }
@@ -235,15 +250,15 @@ static void launch_lru_time(int time_type, dim3 grid, hipStream_t s, const void 
                             int64_t idx_hs, int K, int64_t P, int n_hbm, int32_t *step, int bump,
                             void *time, int64_t time_hs, void *d2h, int64_t d2h_hs, void *h2d,
                             int64_t h2d_hs, uint8_t *hit, int32_t *mp, int32_t *ms, int32_t *mc,
-                            int32_t *ticket, int serial) {
+                            int32_t *se, int32_t *ticket, int serial) {
   if (time_type == DA_TIME_F32)
     hipLaunchKernelGGL((lru_update_kernel<IdxT, MapT, float>), grid, dim3(kSelThreads), 0, s,
                        (const IdxT *)idx, idx_hs, K, P, n_hbm, step, bump, (float *)time, time_hs,
-                       (MapT *)d2h, d2h_hs, (MapT *)h2d, h2d_hs, hit, mp, ms, mc, ticket, serial);
+                       (MapT *)d2h, d2h_hs, (MapT *)h2d, h2d_hs, hit, mp, ms, mc, se, ticket, serial);
   else
     hipLaunchKernelGGL((lru_update_kernel<IdxT, MapT, int32_t>), grid, dim3(kSelThreads), 0, s,
                        (const IdxT *)idx, idx_hs, K, P, n_hbm, step, bump, (int32_t *)time,
-                       time_hs, (MapT *)d2h, d2h_hs, (MapT *)h2d, h2d_hs, hit, mp, ms, mc, ticket,
+                       time_hs, (MapT *)d2h, d2h_hs, (MapT *)h2d, h2d_hs, hit, mp, ms, mc, se, ticket,
                        serial);
 }
 
@@ -257,8 +272,8 @@ extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_i
                              int64_t time_head_stride, int time_type, void *d2h,
                              int64_t d2h_head_stride, void *h2d, int64_t h2d_head_stride,
                              int map_itype, uint8_t *hit_mask, int32_t *miss_page,
-                             int32_t *miss_slot, int32_t *miss_count, void *workspace,
-                             size_t workspace_bytes, void *stream) {
+                             int32_t *miss_slot, int32_t *miss_count, int32_t *slot_epoch,
+                             void *workspace, size_t workspace_bytes, void *stream) {
   using namespace da;
   DA_REQUIRE(n_kv_heads >= 0 && k >= 0 && n_dram_pages >= 0 && n_hbm_pages >= 0,
              "da_lru_update: bad geometry (heads %d k %d pages %lld slots %d)", n_kv_heads, k,
@@ -287,7 +302,7 @@ extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_i
 #define DA_LRU_ARGS                                                                          \
   time_type, grid, s, idx, idx_head_stride, k, n_dram_pages, n_hbm_pages, step, bump_step,   \
       access_time, time_head_stride, d2h, d2h_head_stride, h2d, h2d_head_stride, hit_mask,   \
-      miss_page, miss_slot, miss_count, ticket, serial
+      miss_page, miss_slot, miss_count, slot_epoch, ticket, serial
   if (idx_itype == DA_I64 && map_itype == DA_I64)
     launch_lru_time<int64_t, int64_t>(DA_LRU_ARGS);
   else if (idx_itype == DA_I64)
@@ -316,7 +331,11 @@ extern "C" int da_pages_gather(const void *dram, int64_t dram_head_stride_bytes,
                  (uintptr_t)hbm % 16 == 0,
              "da_pages_gather: pages must be 16-byte aligned multiples of 16 bytes");
   DA_REQUIRE(n_kv_heads <= 65535, "da_pages_gather: too many heads");
-  const int per_head = k < 128 ? k : 128;
+  // Few, fat workgroups: ~32 blocks (16 KiB of reads in flight each) already
+  // saturate the host link, and more concurrent page streams only lower it.
+  int cap = 32 / n_kv_heads;
+  if (cap < 1) cap = 1;
+  const int per_head = k < cap ? k : cap;
   dim3 grid(per_head, n_kv_heads);
   hipLaunchKernelGGL(pages_gather_kernel, grid, dim3(256), 0, (hipStream_t)stream,
                      (const char *)dram, dram_head_stride_bytes, dram_page_stride_bytes,

@@ -23,6 +23,46 @@ __device__ __forceinline__ float bound_term(float q, float mn, float mx) {
   return round_to<T>(fmaxf(q * mn, q * mx));
 }
 
+// Sum of the V bound terms of one 16-byte lane slice.  For 16-bit inputs two
+// maxima are rounded by one packed convert and added to the fp32 accumulator
+// by a dot product with (1, 1): rounding and accumulation in two instructions.
+template <typename T>
+__device__ __forceinline__ float slice_bound(const float *q, const float *mn, const float *mx);
+template <>
+__device__ __forceinline__ float slice_bound<F32>(const float *q, const float *mn,
+                                                  const float *mx) {
+  float a = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a += fmaxf(q[i] * mn[i], q[i] * mx[i]);
+  return a;
+}
+template <>
+__device__ __forceinline__ float slice_bound<BF16>(const float *q, const float *mn,
+                                                   const float *mx) {
+  const bf16x2 ones = as_bf16x2(0x3f803f80u);
+  float a = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i += 2) {
+    const uint32_t pair = pack_bf16(fmaxf(q[i] * mn[i], q[i] * mx[i]),
+                                    fmaxf(q[i + 1] * mn[i + 1], q[i + 1] * mx[i + 1]));
+    a = __builtin_amdgcn_fdot2_f32_bf16(as_bf16x2(pair), ones, a, false);
+  }
+  return a;
+}
+template <>
+__device__ __forceinline__ float slice_bound<F16>(const float *q, const float *mn,
+                                                  const float *mx) {
+  const f16x2 ones = as_f16x2(0x3c003c00u);
+  float a = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i += 2) {
+    const uint32_t pair = pack_f16(fmaxf(q[i] * mn[i], q[i] * mx[i]),
+                                   fmaxf(q[i + 1] * mn[i + 1], q[i + 1] * mx[i + 1]));
+    a = __builtin_amdgcn_fdot2(as_f16x2(pair), ones, a, false);
+  }
+  return a;
+}
+
 template <typename T, int kLanes, int kRows, int kUnroll, typename OutT>
 __global__ void __launch_bounds__(256)
 page_score_vec_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t q_head_stride,
@@ -68,10 +108,7 @@ page_score_vec_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t 
     float acc[kRows];
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
-      float a = 0.f;
-#pragma unroll
-      for (int i = 0; i < V; ++i) a += bound_term<T>(qf[r][i], fmin_[i], fmax_[i]);
-      acc[r] = group_sum<kLanes>(a);
+      acc[r] = group_sum<kLanes>(slice_bound<T>(qf[r], fmin_, fmax_));
     }
     const int64_t p = p_first + u * kGroups + g;
     if (p < n_pages) {

@@ -11,7 +11,20 @@ namespace da {
 
 struct ScoreKey {
   const float *row;
+  bool aligned;  // row starts on a 16-byte boundary
   __device__ __forceinline__ uint32_t operator()(int i) const { return float_order_key(row[i]); }
+  __device__ __forceinline__ void load4(int i, uint32_t *k) const {
+    float4 v;
+    if (aligned) {
+      v = *(const float4 *)(row + i);
+    } else {
+      v = make_float4(row[i], row[i + 1], row[i + 2], row[i + 3]);
+    }
+    k[0] = float_order_key(v.x);
+    k[1] = float_order_key(v.y);
+    k[2] = float_order_key(v.z);
+    k[3] = float_order_key(v.w);
+  }
 };
 
 template <typename IdxT>
@@ -22,10 +35,11 @@ topk_pages_kernel(const float *__restrict__ scores, int64_t row_stride, int64_t 
   __shared__ SelectShared sm;
   const int n = blockIdx.x;  // score row (query row)
   const int h = blockIdx.y;
-  ScoreKey key{scores + n * row_stride + h * head_stride};
-  select_sorted(key, n_pages, kp, sm);
+  const float *row = scores + n * row_stride + h * head_stride;
+  ScoreKey key{row, ((uintptr_t)row & 15) == 0};
+  const uint32_t *best = select_sorted(key, n_pages, kp, sm);
   IdxT *dst = out + (n / rep) * out_seq_stride + h * out_head_stride + (n % rep) * out_rep_stride;
-  for (int j = threadIdx.x; j < kp; j += kSelThreads) dst[j] = (IdxT)sel_index(sm.sel[j]);
+  for (int j = threadIdx.x; j < kp; j += kSelThreads) dst[j] = (IdxT)best[j];
 }
 
 }  // namespace da

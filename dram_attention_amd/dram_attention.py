@@ -9,6 +9,7 @@ start_pos, stage)`` keep their meaning and error behaviour.
 
 from __future__ import annotations
 
+import ctypes
 import math
 
 import torch
@@ -16,6 +17,38 @@ import torch.nn.functional as F
 
 from . import _lib
 from .lru_cache import DummyCache, LRUCache
+
+
+class PagedPrefix:
+    """Says that the prefix handed to :func:`decode_attention` is the slot array of
+    an LRU page cache whose page stream for this step may still be running.
+
+    phase 1 attends over the local window and every slot that keeps its page,
+    phase 2 (after the stream has finished) over the re-assigned slots and writes
+    the output, phase 3 does both at once."""
+
+    def __init__(self, page_size: int, scratch, current_step: torch.Tensor, phase: int):
+        self.page_size = page_size
+        self.scratch = scratch
+        self.current_step = current_step
+        self.phase = phase
+
+    def as_struct(self) -> "_lib.PagedOverlap":
+        s = self.scratch
+        return _lib.PagedOverlap(
+            page_size=self.page_size, phase=self.phase, slot_epoch=s.slot_epoch.data_ptr(),
+            slot_epoch_head_stride=s.slot_epoch.stride(0), epoch=self.current_step.data_ptr(),
+            miss_slot=s.miss_slot.data_ptr(), miss_count=s.miss_count.data_ptr(),
+            miss_capacity=s.miss_slot.shape[1])
+
+
+def attention_workspace(Hq: int, Hkv: int, D: int, dtype: torch.dtype, p_len: int, capacity: int,
+                        miss_tokens: int, device) -> torch.Tensor:
+    need = _lib.load().da_decode_attention_workspace_bytes(
+        Hq, Hkv, D, _lib.dtype_code(dtype), p_len, capacity, miss_tokens)
+    if need == 0:
+        raise RuntimeError(f"decode attention does not cover head_dim={D} dtype={dtype}")
+    return torch.empty((need + 3) // 4, dtype=torch.float32, device=device)
 
 
 def decode_attention(
@@ -32,6 +65,7 @@ def decode_attention(
     out: torch.Tensor | None = None,
     lse: torch.Tensor | None = None,
     scale: float | None = None,
+    paged: PagedPrefix | None = None,
 ) -> torch.Tensor:
     """One query token against [prefix ++ cache rows 0..cache_len ++ new token].
 
@@ -39,6 +73,8 @@ def decode_attention(
     cache_k/v (capacity, Hkv, D); cache_len an int or a one-element int32 GPU
     tensor; new_k/new_v (Hkv, D) are appended at row cache_len (or None).
     Returns (Hq, D) in xq.dtype; fills ``lse`` (Hq, fp32) when given.
+    With ``paged`` the work is split around a concurrent page stream; the same
+    workspace and ``out`` must be passed to both phases.
     """
     Hq, D = xq.shape
     Hkv = cache_k.shape[1]
@@ -49,11 +85,10 @@ def decode_attention(
     capacity = cache_k.shape[0]
     if out is None:
         out = torch.empty(Hq, D, dtype=xq.dtype, device=xq.device)
-    need = lib.da_decode_attention_workspace_bytes(Hq, Hkv, D, dt, p_len, capacity)
-    if need == 0:
-        raise RuntimeError(f"decode attention does not cover head_dim={D} dtype={xq.dtype}")
-    if workspace is None or workspace.numel() * workspace.element_size() < need:
-        workspace = torch.empty((need + 3) // 4, dtype=torch.float32, device=xq.device)
+    if workspace is None:
+        miss_tokens = paged.scratch.miss_slot.shape[1] * paged.page_size if paged else 0
+        workspace = attention_workspace(Hq, Hkv, D, xq.dtype, p_len, capacity, miss_tokens,
+                                        xq.device)
     if isinstance(cache_len, torch.Tensor):
         _lib.require_gpu(cache_len, "cache_len")
         if cache_len.dtype != torch.int32:
@@ -66,8 +101,9 @@ def decode_attention(
     for t in (xq, prefix_k, prefix_v, cache_k, cache_v, new_k, new_v):
         if t is not None and t.numel() and t.stride(-1) != 1:
             raise ValueError("head_dim must be the dense axis of every operand")
+    overlap = paged.as_struct() if paged is not None else None
     _lib.check(
-        lib.da_decode_attention(
+        lib.da_decode_attention_paged(
             xq.data_ptr(), xq.stride(0), Hq, Hkv, D, dt,
             prefix_k.data_ptr() if p_len else None, prefix_v.data_ptr() if p_len else None,
             prefix_k.stride(1) if p_len else 0, prefix_k.stride(0) if p_len else 0, p_len,
@@ -79,6 +115,7 @@ def decode_attention(
             scale, out.data_ptr(), out.stride(0),
             lse.data_ptr() if lse is not None else None,
             workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+            ctypes.byref(overlap) if overlap is not None else None,
             _lib.stream_ptr(xq.device),
         ),
         "da_decode_attention",
@@ -155,6 +192,9 @@ class DRAMAttention(torch.nn.Module):
         self.register_buffer("cache_k", torch.zeros(cache_shape, device=device, dtype=dtype))
         self.register_buffer("cache_v", torch.zeros(cache_shape, device=device, dtype=dtype))
         self._workspace = None
+        self._side_stream = None
+        # stream missed pages on a side stream underneath the attention pass
+        self.overlap_page_stream = True
 
     def init_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor):
         """Split the prompt's (1,S,Hkv,D) keys/values into the paged prefix and the
@@ -195,25 +235,54 @@ class DRAMAttention(torch.nn.Module):
             raise RuntimeError(f"Unsupported stage: {stage}")
 
     def _generate(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, start_pos):
-        """One decode step: page in what the query needs, then one attention pass
-        over resident pages, local window and the new token (appended in place)."""
+        """One decode step: select pages, update the LRU, then one attention pass
+        over resident pages, local window and the new token (appended in place).
+        The missed pages stream in on a side stream while attention already
+        covers the local window and every slot that keeps its page."""
         bsz, seqlen, Hq, D = xq.shape
         if seqlen != 1:
             raise RuntimeError("generate handles one token per call")
-        prefix_k, prefix_v = self.lru_cache.get_kv_cache_(xq)
         if isinstance(start_pos, torch.Tensor):
             cache_len = (start_pos - self.dram_kv_cache_size).to(torch.int32).reshape(1)
         else:
             cache_len = int(start_pos) - self.dram_kv_cache_size
-        if self._workspace is None:
-            lib = _lib.load()
-            need = lib.da_decode_attention_workspace_bytes(
-                Hq, self.n_kv_heads, D, _lib.dtype_code(xq.dtype), prefix_k.shape[1],
-                self.cache_k.shape[1])
-            self._workspace = torch.empty((need + 3) // 4, dtype=torch.float32, device=xq.device)
         out = torch.empty(1, 1, Hq, D, dtype=xq.dtype, device=xq.device)
-        decode_attention(
-            xq[0, 0], prefix_k, prefix_v, self.cache_k[0], self.cache_v[0], cache_len,
-            xk[0, 0], xv[0, 0], workspace=self._workspace, out=out[0, 0],
-        )
+        lru = self.lru_cache
+        if not isinstance(lru, LRUCache):
+            prefix_k, prefix_v = lru.get_kv_cache_(xq)
+            if self._workspace is None:
+                self._workspace = attention_workspace(Hq, self.n_kv_heads, D, xq.dtype,
+                                                      prefix_k.shape[1], self.cache_k.shape[1], 0,
+                                                      xq.device)
+            decode_attention(xq[0, 0], prefix_k, prefix_v, self.cache_k[0], self.cache_v[0],
+                             cache_len, xk[0, 0], xv[0, 0], workspace=self._workspace,
+                             out=out[0, 0])
+            return out
+
+        idx = lru.select_(xq)
+        scratch = lru.update_(idx)
+        prefix_k, prefix_v = lru.views()
+        if self._workspace is None:
+            self._workspace = attention_workspace(
+                Hq, self.n_kv_heads, D, xq.dtype, prefix_k.shape[1], self.cache_k.shape[1],
+                scratch.miss_slot.shape[1] * self.page_size, xq.device)
+        args = (xq[0, 0], prefix_k, prefix_v, self.cache_k[0], self.cache_v[0], cache_len,
+                xk[0, 0], xv[0, 0])
+        if not self.overlap_page_stream:
+            lru.gather_(idx.shape[1])
+            decode_attention(*args, workspace=self._workspace, out=out[0, 0],
+                             paged=PagedPrefix(self.page_size, scratch, lru.current_step, 3))
+            return out
+        main = torch.cuda.current_stream(xq.device)
+        if self._side_stream is None:
+            self._side_stream = torch.cuda.Stream(device=xq.device)
+        side = self._side_stream
+        side.wait_stream(main)                      # the miss list is ready
+        with torch.cuda.stream(side):
+            lru.gather_(idx.shape[1])
+        decode_attention(*args, workspace=self._workspace, out=out[0, 0],
+                         paged=PagedPrefix(self.page_size, scratch, lru.current_step, 1))
+        main.wait_stream(side)                      # the pages have landed
+        decode_attention(*args, workspace=self._workspace, out=out[0, 0],
+                         paged=PagedPrefix(self.page_size, scratch, lru.current_step, 2))
         return out

@@ -12,7 +12,7 @@ from typing import NamedTuple, Optional
 import torch
 
 from . import _lib
-from .lru_kernel import LruScratch, lru_update_and_gather
+from .lru_kernel import LruScratch, lru_update, lru_update_and_gather, pages_gather
 from .topk_selector import IPUpperboundTopKSelector
 
 
@@ -119,7 +119,8 @@ class LRUCache(torch.nn.Module):
     # -- internals ---------------------------------------------------------
     def _scratch_for(self, k: int) -> LruScratch:
         if self._scratch is None or self._scratch.miss_page.shape[1] != max(k, 1):
-            self._scratch = LruScratch.allocate(self.num_kv_heads, k, self.hbm_kv_cache.device)
+            self._scratch = LruScratch.allocate(self.num_kv_heads, k, self.hbm_kv_cache.device,
+                                                self.num_hbm_pages)
         return self._scratch
 
     def _views(self) -> CacheOutput:
@@ -149,13 +150,39 @@ class LRUCache(torch.nn.Module):
         bsz, seq_len, num_q_heads, _ = q.shape
         assert num_q_heads % self.num_kv_heads == 0
         rep = num_q_heads // self.num_kv_heads
+        return self.load_(self.select_(q))
+
+    # -- the same step in separable pieces (used by DRAMAttention to overlap the
+    #    page stream with attention over the slots that keep their page) -------
+    def select_(self, q: torch.Tensor) -> torch.Tensor:
+        """Scores + ordered top-k: the (H, seq_len*rep*k) request list of this step."""
+        bsz, seq_len, num_q_heads, _ = q.shape
+        assert num_q_heads % self.num_kv_heads == 0
+        rep = num_q_heads // self.num_kv_heads
         k = min(self.top_k, self.num_dram_pages)
         total = seq_len * rep * k
         if self._topk_idx is None or self._topk_idx.shape[1] != total:
             self._topk_idx = torch.empty(self.num_kv_heads, total, dtype=torch.int64,
                                          device=q.device)
-        idx = self.top_k_selector.top_k_for_lru(q, k, out=self._topk_idx)
-        return self.load_(idx)
+        return self.top_k_selector.top_k_for_lru(q, k, out=self._topk_idx)
+
+    def update_(self, idx: torch.Tensor) -> LruScratch:
+        """Metadata only: advance the step, touch/evict/assign, emit the miss list."""
+        scratch = self._scratch_for(idx.shape[1])
+        lru_update(self.dram_kv_cache, self.page_access_time, self.dram_page_to_hbm_page_mapping,
+                   self.hbm_page_to_dram_page_mapping, idx, self.current_step, self.hbm_kv_cache,
+                   scratch, bump_step=True)
+        return scratch
+
+    def gather_(self, k: int) -> None:
+        """Stream the pages of the last miss list into their slots (current stream)."""
+        if self._dram_device_ptr is None:
+            self._dram_device_ptr = _lib.device_visible_ptr(self.dram_kv_cache)
+        pages_gather(self.dram_kv_cache, self.hbm_kv_cache, self._scratch, k,
+                     self._dram_device_ptr)
+
+    def views(self) -> CacheOutput:
+        return self._views()
 
     # -- instrumentation (absent from the reference) -------------------------
     def last_miss_counts(self) -> torch.Tensor:

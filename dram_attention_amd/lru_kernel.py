@@ -21,12 +21,15 @@ class LruScratch(NamedTuple):
     miss_count: torch.Tensor  # (H,) int32
     hit_mask: torch.Tensor    # (H, K) uint8: 1 = resident when visited
     workspace: torch.Tensor   # zeroed once; holds the step-bump ticket
+    slot_epoch: torch.Tensor  # (H, N_hbm) int32: step at which a slot was last re-assigned
 
     @staticmethod
-    def allocate(num_heads: int, k: int, device) -> "LruScratch":
+    def allocate(num_heads: int, k: int, device, num_hbm_pages: int = 0) -> "LruScratch":
         lib = _lib.load()
         ws = lib.da_lru_update_workspace_bytes(num_heads, k, 0, 0)
         return LruScratch(
+            slot_epoch=torch.zeros(num_heads, max(num_hbm_pages, 1), dtype=torch.int32,
+                                   device=device),
             miss_page=torch.empty(num_heads, max(k, 1), dtype=torch.int32, device=device),
             miss_slot=torch.empty(num_heads, max(k, 1), dtype=torch.int32, device=device),
             miss_count=torch.zeros(num_heads, dtype=torch.int32, device=device),
@@ -35,7 +38,7 @@ class LruScratch(NamedTuple):
         )
 
 
-def lru_update_and_gather(
+def lru_update(
     dram_kv_cache: torch.Tensor,
     page_access_time: torch.Tensor,
     dram_page_to_hbm_page_mapping: torch.Tensor,
@@ -45,9 +48,9 @@ def lru_update_and_gather(
     hbm_kv_cache: torch.Tensor,
     scratch: LruScratch,
     bump_step: bool,
-    dram_device_ptr: Optional[int] = None,
 ) -> None:
-    """Two launches on the current stream: metadata update, then page gather."""
+    """The metadata half of a step: touch, evict, assign; leaves the miss list in
+    ``scratch`` (one launch on the current stream)."""
     num_heads, num_dram_pages, page_dim = dram_kv_cache.shape
     _, k = topk_dram_page_index.shape
     assert (
@@ -73,9 +76,8 @@ def lru_update_and_gather(
         raise TypeError("DRAM and HBM page stores must share one element type")
     if dram_kv_cache.stride(2) != 1 or hbm_kv_cache.stride(2) != 1:
         raise ValueError("pages must be dense")
-    dev = hbm_kv_cache.device
+    epoch = scratch.slot_epoch if scratch.slot_epoch.shape == (num_heads, num_hbm_pages) else None
     lib = _lib.load()
-    stream = _lib.stream_ptr(dev)
     _lib.check(
         lib.da_lru_update(
             topk_dram_page_index.data_ptr(), topk_dram_page_index.stride(0),
@@ -88,22 +90,52 @@ def lru_update_and_gather(
             _lib.itype_code(dram_page_to_hbm_page_mapping.dtype),
             scratch.hit_mask.data_ptr(), scratch.miss_page.data_ptr(),
             scratch.miss_slot.data_ptr(), scratch.miss_count.data_ptr(),
-            scratch.workspace.data_ptr(), scratch.workspace.numel(), stream,
+            epoch.data_ptr() if epoch is not None else None,
+            scratch.workspace.data_ptr(), scratch.workspace.numel(),
+            _lib.stream_ptr(hbm_kv_cache.device),
         ),
         "da_lru_update",
     )
+
+
+def pages_gather(dram_kv_cache: torch.Tensor, hbm_kv_cache: torch.Tensor, scratch: LruScratch,
+                 k: int, dram_device_ptr: Optional[int] = None) -> None:
+    """The data half: copy every page of the miss list into its slot (one launch
+    on the current stream; the page store may be pinned host memory)."""
+    num_heads, _, page_dim = dram_kv_cache.shape
     if dram_device_ptr is None:
         dram_device_ptr = _lib.device_visible_ptr(dram_kv_cache)
     esz = dram_kv_cache.element_size()
+    lib = _lib.load()
     _lib.check(
         lib.da_pages_gather(
             dram_device_ptr, dram_kv_cache.stride(0) * esz, dram_kv_cache.stride(1) * esz,
             hbm_kv_cache.data_ptr(), hbm_kv_cache.stride(0) * esz, hbm_kv_cache.stride(1) * esz,
             page_dim * esz, scratch.miss_page.data_ptr(), scratch.miss_slot.data_ptr(),
-            scratch.miss_count.data_ptr(), num_heads, k, stream,
+            scratch.miss_count.data_ptr(), num_heads, k, _lib.stream_ptr(hbm_kv_cache.device),
         ),
         "da_pages_gather",
     )
+
+
+def lru_update_and_gather(
+    dram_kv_cache: torch.Tensor,
+    page_access_time: torch.Tensor,
+    dram_page_to_hbm_page_mapping: torch.Tensor,
+    hbm_page_to_dram_page_mapping: torch.Tensor,
+    topk_dram_page_index: torch.Tensor,
+    current_step: torch.Tensor,
+    hbm_kv_cache: torch.Tensor,
+    scratch: LruScratch,
+    bump_step: bool,
+    dram_device_ptr: Optional[int] = None,
+) -> None:
+    """Two launches on the current stream: metadata update, then page gather."""
+    lru_update(dram_kv_cache, page_access_time, dram_page_to_hbm_page_mapping,
+               hbm_page_to_dram_page_mapping, topk_dram_page_index, current_step, hbm_kv_cache,
+               scratch, bump_step)
+    pages_gather(dram_kv_cache, hbm_kv_cache, scratch, topk_dram_page_index.shape[1],
+                 dram_device_ptr)
 
 
 def load_lru_cache_(

@@ -124,6 +124,9 @@ int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
  *   hit_mask     : optional (Hkv, K) bytes, 1 = page was resident when visited
  *   miss_page/miss_slot : (Hkv, K) int32, the i-th distinct missed page of a
  *                  head and the slot it was given; miss_count : (Hkv) int32
+ *   slot_epoch   : optional (Hkv, N_hbm) int32; a slot handed to a missed page
+ *                  gets the step value, so a later kernel can tell which slots
+ *                  the page stream of this step is (still) writing
  * The end state equals the reference's serial walk for every input; K <=
  * N_hbm runs fully parallel, K > N_hbm falls back to one serial lane per head.
  * A miss_slot of -1 marks an entry whose slot was re-assigned later in the
@@ -139,8 +142,8 @@ int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_itype,
                   int64_t time_head_stride, int time_type, void *d2h,
                   int64_t d2h_head_stride, void *h2d, int64_t h2d_head_stride,
                   int map_itype, uint8_t *hit_mask, int32_t *miss_page,
-                  int32_t *miss_slot, int32_t *miss_count, void *workspace,
-                  size_t workspace_bytes, void *stream);
+                  int32_t *miss_slot, int32_t *miss_count, int32_t *slot_epoch,
+                  void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Subsystem 4b — stream the missed pages into their HBM slots.
@@ -175,12 +178,14 @@ int da_pages_gather(const void *dram, int64_t dram_head_stride_bytes,
  *   new_k, new_v : (Hkv, D) of the current token (head stride new_head_stride),
  *                  or NULL to attend over the c_len cached rows only
  *   out          : (Hq, D) in `dtype`;  lse_out : optional (Hq) fp32, natural log
- * fp32 accumulation throughout; 16-bit inputs use packed dot products, so
- * probabilities are rounded to the input type before they weight the values
- * (as flash-attn does).
+ * fp32 accumulation throughout; 16-bit query/key products use packed dot
+ * instructions.
+ * workspace: da_decode_attention_workspace_bytes(...) bytes, 16-byte aligned, no
+ * initial state; `miss_tokens` is 0 here (see da_decode_attention_paged).
  */
 size_t da_decode_attention_workspace_bytes(int n_q_heads, int n_kv_heads, int head_dim,
-                                           int dtype, int64_t p_len, int64_t c_capacity);
+                                           int dtype, int64_t p_len, int64_t c_capacity,
+                                           int64_t miss_tokens);
 int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
                         int n_kv_heads, int head_dim, int dtype, const void *pk,
                         const void *pv, int64_t p_tok_stride, int64_t p_head_stride,
@@ -190,6 +195,42 @@ int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
                         int64_t new_head_stride, float scale, void *out,
                         int64_t out_head_stride, float *lse_out, void *workspace,
                         size_t workspace_bytes, void *stream);
+
+/*
+ * The same attention when the prefix is the slot array of the LRU page cache
+ * and the missed pages of this step are streamed in concurrently on another
+ * stream (no counterpart in the reference, whose page copies and attention are
+ * serialised on one stream, dram_attention/dram_attention.py:161-172).
+ *   phase 1 : local segment + every slot whose slot_epoch differs from *epoch;
+ *             may run while da_pages_gather is still writing the other slots
+ *   phase 2 : the slots listed in miss_slot[h, 0..miss_count[h]) (entries of -1
+ *             are skipped), then the merge that writes `out`; issue it after the
+ *             page stream has completed
+ *   phase 3 : both, back to back (the page stream must have completed)
+ * The two phases of a step must be given identical arguments otherwise.  The
+ * workspace needs miss_tokens = miss_capacity * page_size.
+ */
+typedef struct da_paged_overlap {
+  int32_t page_size;              /* tokens per slot; p_len = slots * page_size */
+  int32_t phase;                  /* 1, 2 or 3 */
+  const int32_t *slot_epoch;      /* (Hkv, slots), written by da_lru_update */
+  int64_t slot_epoch_head_stride; /* elements */
+  const int32_t *epoch;           /* the LRU step counter after da_lru_update */
+  const int32_t *miss_slot;       /* (Hkv, miss_capacity) */
+  const int32_t *miss_count;      /* (Hkv) */
+  int32_t miss_capacity;
+} da_paged_overlap;
+
+int da_decode_attention_paged(const void *q, int64_t q_head_stride, int n_q_heads,
+                              int n_kv_heads, int head_dim, int dtype, const void *pk,
+                              const void *pv, int64_t p_tok_stride, int64_t p_head_stride,
+                              int64_t p_len, void *ck, void *cv, int64_t c_tok_stride,
+                              int64_t c_head_stride, int64_t c_capacity, int64_t c_len,
+                              const int32_t *c_len_dev, const void *new_k, const void *new_v,
+                              int64_t new_head_stride, float scale, void *out,
+                              int64_t out_head_stride, float *lse_out, void *workspace,
+                              size_t workspace_bytes, const da_paged_overlap *overlap,
+                              void *stream);
 
 #ifdef __cplusplus
 }

@@ -210,6 +210,39 @@ def test_decode_parity_device_side_position_and_rep8():
     run_parity(w, 2, w.steps, atol=2e-2, rtol=1e-2, device_pos=True)
 
 
+def test_page_stream_overlap_changes_nothing():
+    """Attention issued around a concurrent page stream (two phases, side stream)
+    gives the bits of the serialised order, and both agree with one plain pass."""
+    from dram_attention_amd import DRAMAttention, decode_attention
+
+    w = WORKLOADS["128k"].scaled(dram_tokens=16384, local_cache=1024, lru_tokens=4096,
+                                 top_k_tokens=1024, steps=5)
+    prompt = make_prompt(w, 4)
+    mods = []
+    for overlap in (True, False):
+        m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, 16, w.top_k_tokens, w.n_kv_heads,
+                          w.head_dim, device=DEV, dtype=w.dtype)
+        m.overlap_page_stream = overlap
+        m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+        mods.append(m)
+    inputs = DecodeInputs(w, prompt.q0, 4)
+    for t in range(w.steps):
+        xq, xk, xv = (x.to(DEV) for x in inputs.next())
+        a = mods[0](xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
+        b = mods[1](xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
+        torch.cuda.synchronize()
+        assert mods[0].lru_cache.last_miss_counts().sum().item() > 0
+        assert same(a, b), f"step {t}"
+        assert same(mods[0].lru_cache.hbm_kv_cache, mods[1].lru_cache.hbm_kv_cache)
+        # one plain pass over the final slot contents (the token is already appended)
+        lru = mods[1].lru_cache
+        pk, pv = lru.views()
+        c = w.prompt_tokens + t - w.dram_tokens
+        plain = decode_attention(xq[0, 0], pk, pv, mods[1].cache_k[0], mods[1].cache_v[0], c + 1,
+                                 None, None)
+        assert close(plain, b[0, 0], 1e-2, 1e-2)
+
+
 def test_static_prefix_equals_full_attention():
     """Prefix within the HBM budget: the static cache path is dense attention over
     the whole sequence (the 32K configuration through init_cache)."""

@@ -32,9 +32,10 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_workspace_queries_need_no_gpu(lib):
-    n = lib.da_decode_attention_workspace_bytes(32, 8, 128, 2, 32768, 4160)
+    n = lib.da_decode_attention_workspace_bytes(32, 8, 128, 2, 32768, 4160, 0)
     assert n > 32 * 130 * 4
-    assert lib.da_decode_attention_workspace_bytes(32, 8, 24, 2, 1024, 64) == 0   # unsupported dim
+    assert lib.da_decode_attention_workspace_bytes(32, 8, 128, 2, 32768, 4160, 16384) > n
+    assert lib.da_decode_attention_workspace_bytes(32, 8, 24, 2, 1024, 64, 0) == 0   # unsupported dim
     assert lib.da_lru_update_workspace_bytes(8, 1024, 8192, 2048) >= 4
 
 
