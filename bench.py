@@ -1,18 +1,19 @@
 #!/usr/bin/env python3
 """Decode-step benchmark of the DRAM Attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 128k] [--eager]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 128k] [--eager] [--no-overlap]
 
 A step is one `generate` call of one attention layer: page scoring, ordered
 top-k, LRU update, streaming of missed pages from pinned host DRAM, and decode
 attention over the resident pages + local window + new token.  Inputs of all
 steps are staged in HBM before the clock starts.  By default the step is
 captured once into a HIP graph (position and LRU step live on the device) and
-replayed; --eager issues the launches from Python every step.
+replayed; --eager issues the launches from Python every step; --no-overlap
+keeps the page stream and attention on one stream.
 
-Prints ONE JSON line: the BASELINE metric plus `roofline` (dominant kernel,
-timed live with events on the launch stream) and `cpu_baseline` (the CPU oracle
-timed on this box's host cores on a bounded sample of the same workload).
+Prints ONE JSON line: the BASELINE metric plus `roofline` (the dominant HBM
+kernel, timed live with events on the launch stream) and `cpu_baseline` (the CPU
+oracle timed on this box's host cores on a bounded sample of the same workload).
 """
 
 from __future__ import annotations
@@ -29,6 +30,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+WORKLOAD_INDEX = {"cpu": 0, "32k": 1, "128k": 2, "1m": 4}
 
 
 def parse_args():
@@ -36,18 +38,22 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="128k", choices=["cpu", "32k", "128k", "1m"])
+    ap.add_argument("--workload", default="128k", choices=sorted(WORKLOAD_INDEX))
     ap.add_argument("--eager", action="store_true", help="no HIP graph: launch from Python each step")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="page stream and attention serialised on one stream")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-steps", type=int, default=8, help="steps of the CPU oracle to time (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=16, help="extra steps timed per kernel with events")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 128 MiB device copy (reference point for HBM traffic counters)")
     return ap.parse_args()
 
 
 class Layer:
     """One attention layer set up on the workload, plus the staged step inputs."""
 
-    def __init__(self, w, seed, total_steps, dev):
+    def __init__(self, w, seed, total_steps, dev, overlap):
         from dram_attention_amd import DRAMAttention
         from dram_attention_amd.synthetic import DecodeInputs, make_prompt
 
@@ -58,6 +64,7 @@ class Layer:
                                local_cache_size=w.local_cache, page_size=w.page_size,
                                top_k=w.top_k_tokens, n_kv_heads=w.n_kv_heads, head_dim=w.head_dim,
                                device=dev, dtype=w.dtype)
+        self.m.overlap_page_stream = overlap
         self.m.init_cache(prompt.k.to(dev), prompt.v.to(dev))
         inputs = DecodeInputs(w, prompt.q0, seed)
         qs, ks, vs = zip(*(inputs.next() for _ in range(total_steps)))
@@ -65,19 +72,26 @@ class Layer:
         self.qs = torch.cat(qs).to(dev)   # (T, 1, Hq, D)
         self.ks = torch.cat(ks).to(dev)
         self.vs = torch.cat(vs).to(dev)
-        self.t_dev = torch.zeros(1, dtype=torch.int64, device=dev)          # step index
-        self.pos_dev = torch.full((1,), w.prompt_tokens, dtype=torch.int32, device=dev)
+        # What the rest of a model would hand to the layer each step, staged as one
+        # row per step: [q heads | k heads | v heads], fetched by one index_select.
+        Hq, Hkv, D = w.n_q_heads, w.n_kv_heads, w.head_dim
+        self.qkv = torch.cat([self.qs.view(total_steps, Hq * D), self.ks.view(total_steps, Hkv * D),
+                              self.vs.view(total_steps, Hkv * D)], dim=1).contiguous()
+        # [step index, position]: both advance with a single increment kernel
+        self.ctr = torch.tensor([0, w.prompt_tokens], dtype=torch.int32, device=dev)
+        self.t_dev, self.pos_dev = self.ctr[0:1], self.ctr[1:2]
         self.out = None
 
     def step_from_device_state(self):
         """One decode step driven entirely by device-resident counters."""
-        m = self.m
-        xq = self.qs.index_select(0, self.t_dev)
-        xk = self.ks.index_select(0, self.t_dev)
-        xv = self.vs.index_select(0, self.t_dev)
+        w, m = self.w, self.m
+        Hq, Hkv, D = w.n_q_heads, w.n_kv_heads, w.head_dim
+        row = self.qkv.index_select(0, self.t_dev)[0]
+        xq = row[: Hq * D].view(1, 1, Hq, D)
+        xk = row[Hq * D:(Hq + Hkv) * D].view(1, 1, Hkv, D)
+        xv = row[(Hq + Hkv) * D:].view(1, 1, Hkv, D)
         self.out = m(xq, xk, xv, start_pos=self.pos_dev, stage="generate")
-        self.t_dev += 1
-        self.pos_dev += 1
+        self.ctr += 1
         return self.out
 
 
@@ -89,42 +103,96 @@ def algorithmic_bytes(w, local_rows):
 
 
 def time_kernels(layer, steps):
-    """Per-entry-point GPU time, events recorded on the stream the kernels run on."""
-    from dram_attention_amd.dram_attention import decode_attention
+    """Per-kernel GPU time over `steps` further decode steps, issued one launch at a
+    time on the current stream with an event on either side.  A short busy kernel
+    goes first so that both events and the launch are queued before the GPU gets
+    to them: the interval is the kernel, not the host's launch latency.  The page
+    stream runs to completion before attention here (no overlap), so each kernel
+    is seen alone."""
+    from dram_attention_amd.dram_attention import PagedPrefix, decode_attention
 
-    m, lru = layer.m, layer.m.lru_cache
-    names = ("page_score", "topk_pages", "lru_update+pages_gather", "decode_attention")
+    from dram_attention_amd import LRUCache
+
+    m, lru, w = layer.m, layer.m.lru_cache, layer.w
+    names = ("page_score", "topk_pages", "lru_update", "pages_gather", "decode_attention_split",
+             "decode_attention_tail+merge")
     acc = {n: 0.0 for n in names}
-    misses = 0
-    local_rows = []
+    misses, local_rows = 0, []
+    if not isinstance(lru, LRUCache):
+        # prefix within the HBM budget: no paging, the step is one attention pass
+        for _ in range(steps):
+            t = int(layer.t_dev.item())
+            xq, xk, xv = layer.qs[t:t + 1], layer.ks[t:t + 1], layer.vs[t:t + 1]
+            pk, pv = lru.get_kv_cache_(xq)
+            c_len = int(layer.pos_dev.item()) - m.dram_kv_cache_size
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda._sleep(2_000_000)
+            e0.record()
+            decode_attention(xq[0, 0], pk, pv, m.cache_k[0], m.cache_v[0], c_len, xk[0, 0],
+                             xv[0, 0], workspace=m._workspace)
+            e1.record()
+            torch.cuda.synchronize()
+            acc["decode_attention_split"] += e0.elapsed_time(e1)   # includes its merge launch
+            local_rows.append(c_len)
+            layer.ctr += 1
+        return ({"decode_attention_split": acc["decode_attention_split"] / steps * 1e3}, 0.0,
+                sum(local_rows) / len(local_rows))
+
+    def timed(name, fn, repeat=8):
+        """`repeat` back-to-back launches between one pair of events (the kernels
+        timed this way are idempotent); the interval / repeat is one launch."""
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda._sleep(2_000_000)  # GPU busy time: the whole batch is queued behind it
+        e0.record()
+        for _ in range(repeat):
+            r = fn()
+        e1.record()
+        pending.append((name, e0, e1, repeat))
+        return r
+
     for _ in range(steps):
+        pending = []
         t = int(layer.t_dev.item())
         xq, xk, xv = layer.qs[t:t + 1], layer.ks[t:t + 1], layer.vs[t:t + 1]
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(5)]
         sel = lru.top_k_selector
         k = min(lru.top_k, lru.num_dram_pages)
-        ev[0].record()
-        scores = sel.scores(xq)
-        ev[1].record()
         from dram_attention_amd.topk_selector import topk_pages
+        scores = timed("page_score", lambda: sel.scores(xq))
         idx = lru._topk_idx
-        topk_pages(scores, layer.w.rep, k, idx, layer.w.rep * k, idx.shape[1], k)
-        ev[2].record()
-        pk, pv = lru.load_(idx)
-        ev[3].record()
+        timed("topk_pages", lambda: topk_pages(scores, w.rep, k, idx, w.rep * k, idx.shape[1], k))
+        scratch = timed("lru_update", lambda: lru.update_(idx), repeat=1)   # mutates its state
+        timed("pages_gather", lambda: lru.gather_(idx.shape[1]))
+        pk, pv = lru.views()
         c_len = int(layer.pos_dev.item()) - m.dram_kv_cache_size
-        out = decode_attention(xq[0, 0], pk, pv, m.cache_k[0], m.cache_v[0], c_len, xk[0, 0],
-                               xv[0, 0], workspace=m._workspace)
-        ev[4].record()
+        args = (xq[0, 0], pk, pv, m.cache_k[0], m.cache_v[0], c_len, xk[0, 0], xv[0, 0])
+        out = torch.empty(w.n_q_heads, w.head_dim, dtype=w.dtype, device=xq.device)
+        timed("decode_attention_split", lambda: decode_attention(
+            *args, workspace=m._workspace, out=out,
+            paged=PagedPrefix(w.page_size, scratch, lru.current_step, 1)))
+        timed("decode_attention_tail+merge", lambda: decode_attention(
+            *args, workspace=m._workspace, out=out,
+            paged=PagedPrefix(w.page_size, scratch, lru.current_step, 2)))
         torch.cuda.synchronize()
-        for i, n in enumerate(names):
-            acc[n] += ev[i].elapsed_time(ev[i + 1])
+        for name, e0, e1, repeat in pending:
+            acc[name] += e0.elapsed_time(e1) / repeat
         misses += int(lru.last_miss_counts().sum().item())
         local_rows.append(c_len)
-        layer.t_dev += 1
-        layer.pos_dev += 1
+        layer.ctr += 1
     return ({n: v / steps * 1e3 for n, v in acc.items()},  # microseconds
             misses / steps, sum(local_rows) / len(local_rows))
+
+
+def host_link_gbps(dev, mb=64, reps=5):
+    """Pinned host -> HBM copy rate of the box (hipMemcpyAsync through torch)."""
+    src = torch.empty(mb << 20, dtype=torch.uint8).pin_memory()
+    dst = torch.empty(mb << 20, dtype=torch.uint8, device=dev)
+    dst.copy_(src, non_blocking=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        dst.copy_(src, non_blocking=True)
+    torch.cuda.synchronize()
+    return reps * (mb << 20) / (time.perf_counter() - t0) / 1e9
 
 
 def cpu_baseline(w, layer, steps):
@@ -163,7 +231,7 @@ def main():
     torch.cuda.set_device(dev)
     w = WORKLOADS[args.workload]
     total = args.warmup + args.steps + args.profile_steps + 4
-    layer = Layer(w, args.seed, total, dev)
+    layer = Layer(w, args.seed, total, dev, overlap=not args.no_overlap)
     torch.cuda.synchronize()
 
     # -- warm-up (also resolves the pinned-host device address before any capture)
@@ -202,10 +270,21 @@ def main():
     # -- per-kernel pass and traffic counters
     kernel_us, miss_per_step, local_rows = time_kernels(layer, args.profile_steps)
     score_b, attn_b = algorithmic_bytes(w, local_rows)
-    attn_us = kernel_us["decode_attention"]
+    attn_us = kernel_us["decode_attention_split"]
     achieved = attn_b / (attn_us * 1e-6) / 1e9
     requests = w.n_kv_heads * w.rep * w.pages_per_q_head
     page_bytes = w.page_size * 2 * w.head_dim * torch.empty(0, dtype=w.dtype).element_size()
+    link = host_link_gbps(dev)
+    if args.calibrate_copy:
+        # a plain elementwise kernel of known traffic: reads 128 MiB, writes 128 MiB
+        src = torch.ones(32 << 20, dtype=torch.float32, device=dev)
+        dst = torch.add(src, 1.0)
+        torch.cuda.synchronize()
+        del src, dst
+    stream_gbps = (miss_per_step * page_bytes / (kernel_us["pages_gather"] * 1e-6) / 1e9
+                   if miss_per_step else 0.0)
+    score_gbps = (score_b / (kernel_us["page_score"] * 1e-6) / 1e9
+                  if "page_score" in kernel_us else None)
 
     result = {
         "metric": "decode steps/sec per layer at 128K ctx; scorer+attn HBM GB/s vs peak",
@@ -221,23 +300,27 @@ def main():
         "dtype": {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[w.dtype],
         "data": "synthetic",
         "config": {
-            "workload": f"configs[{['cpu', '32k', '128k', '128k-x32', '1m'].index(w.name)}] {w.name}: "
+            "workload": f"configs[{WORKLOAD_INDEX[w.name]}] {w.name}: "
                         f"1 layer, {w.n_q_heads}q/{w.n_kv_heads}kv heads, D {w.head_dim}, "
                         f"{w.dram_tokens}-token prefix in pinned host DRAM ({w.n_dram_pages} pages/head), "
                         f"local {w.local_cache}, LRU {w.lru_tokens} tokens, top-k {w.top_k_tokens} tokens",
             "launch": "eager" if args.eager else "hip-graph replay",
+            "page_stream": "serialised" if args.no_overlap else "side stream under attention",
             "seed": args.seed,
         },
         "roofline": {
-            "bound": "hbm", "kernel": "decode_attention (split + merge launches)",
+            "bound": "hbm", "kernel": "decode_attention_split_kernel (prefix + local segments)",
             "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
             "algorithmic_bytes": attn_b, "avg_us": attn_us,
         },
         "kernels_us": kernel_us,
-        "page_score_GBps": score_b / (kernel_us["page_score"] * 1e-6) / 1e9,
-        "lru": {"requests_per_step": requests, "distinct_misses_per_step": miss_per_step,
-                "h2d_bytes_per_step": miss_per_step * page_bytes},
+        "page_score_GBps": score_gbps,
+        "page_stream": {"requests_per_step": requests, "distinct_misses_per_step": miss_per_step,
+                        "h2d_bytes_per_step": miss_per_step * page_bytes,
+                        "gather_GBps": stream_gbps, "host_link_memcpy_GBps": link,
+                        "frac_of_link": stream_gbps / link if link else None,
+                        "hit_rate": 1.0 - miss_per_step / requests},
     }
     if args.cpu_steps > 0:
         result["cpu_baseline"] = cpu_baseline(w, layer, args.cpu_steps)

@@ -52,7 +52,7 @@ SIGNATURES = {
     "da_pages_gather": (
         c_int,
         [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
-         c_void_p, c_int, c_int, c_void_p],
+         c_void_p, c_int, c_int, c_int, c_void_p],
     ),
     "da_decode_attention_workspace_bytes": (
         c_size_t, [c_int, c_int, c_int, c_int, c_int64, c_int64, c_int64]),

@@ -25,15 +25,26 @@
 // slots through the miss list and then merges everything.  Both phases are the
 // same kernel; a chunk id says which segment a block works on.
 #include "common.hpp"
+#ifdef DA_TUNE
+#include <stdlib.h>
+#endif
 
 namespace da {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kMinusHuge = -1.0e30f;  // finite stand-in for -inf as a running max
+// The softmax reference m of a lane group is not kept equal to the running
+// maximum: it is only raised when a score exceeds it by more than this many
+// powers of two.  Softmax is shift invariant, so the result is the same; the
+// weights stay below 2^slack, and the register-wide rescale becomes rare.
+constexpr float kRescaleSlack = 8.0f;
 constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = kAttnThreads / 64;
-constexpr int kAttnUnroll = 4;
+#ifndef DA_ATTN_UNROLL
+#define DA_ATTN_UNROLL 4
+#endif
+constexpr int kAttnUnroll = DA_ATTN_UNROLL;  // tokens in flight per lane group (even)
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -63,6 +74,68 @@ __device__ __forceinline__ float dot16<F16>(const u32x4 &q, const u32x4 &k) {
   return a;
 }
 
+// acc[r][:] += p0[r] * v0[:] + p1[r] * v1[:] for the lane's 16-byte value slices
+// of two tokens.  16-bit types interleave the two slices so that one packed dot
+// product per output channel takes both tokens; the probabilities are rounded
+// to the value type for it (as flash-attn does before its P*V product).
+template <typename T, int kRows>
+struct PvPair;
+template <int kRows>
+struct PvPair<F32, kRows> {
+  static __device__ __forceinline__ void run(const u32x4 &v0, const u32x4 &v1, const float *p0,
+                                             const float *p1, float (*acc)[4]) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc[r][i] = fmaf(p1[r], as_f32(v1[i]), fmaf(p0[r], as_f32(v0[i]), acc[r][i]));
+    }
+  }
+};
+template <int kRows>
+struct PvPair<BF16, kRows> {
+  static __device__ __forceinline__ void run(const u32x4 &v0, const u32x4 &v1, const float *p0,
+                                             const float *p1, float (*acc)[8]) {
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      lo[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x05040100u);  // (v0 ch 2i,   v1 ch 2i)
+      hi[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x07060302u);  // (v0 ch 2i+1, v1 ch 2i+1)
+    }
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const bf16x2 pp = as_bf16x2(pack_bf16(p0[r], p1[r]));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[r][2 * i] = __builtin_amdgcn_fdot2_f32_bf16(as_bf16x2(lo[i]), pp, acc[r][2 * i], false);
+        acc[r][2 * i + 1] =
+            __builtin_amdgcn_fdot2_f32_bf16(as_bf16x2(hi[i]), pp, acc[r][2 * i + 1], false);
+      }
+    }
+  }
+};
+template <int kRows>
+struct PvPair<F16, kRows> {
+  static __device__ __forceinline__ void run(const u32x4 &v0, const u32x4 &v1, const float *p0,
+                                             const float *p1, float (*acc)[8]) {
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      lo[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x05040100u);
+      hi[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x07060302u);
+    }
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const f16x2 pp = as_f16x2(pack_f16(p0[r], p1[r]));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[r][2 * i] = __builtin_amdgcn_fdot2(as_f16x2(lo[i]), pp, acc[r][2 * i], false);
+        acc[r][2 * i + 1] = __builtin_amdgcn_fdot2(as_f16x2(hi[i]), pp, acc[r][2 * i + 1], false);
+      }
+    }
+  }
+};
+
 struct AttnArgs {
   const char *q;
   int64_t q_head_stride;  // elements
@@ -75,7 +148,8 @@ struct AttnArgs {
   const char *new_k, *new_v;
   int64_t new_head_stride;
   float scale_log2;  // softmax scale * log2(e)
-  int chunk;         // tokens per block
+  int chunk;         // tokens per block (prefix and local segments)
+  int tail_chunk;    // tokens per block of the tail segment
   // chunk ids: [0, n_pchunks) prefix, [n_pchunks, +n_lchunks) local, then n_tchunks tail
   int n_pchunks, n_lchunks, n_tchunks;
   int chunk_base;  // chunk id of blockIdx.x == 0 in this launch
@@ -84,6 +158,7 @@ struct AttnArgs {
   float *part_acc;  // (chunks, Hq, D)
   // paged prefix with overlap (all null / 0 otherwise)
   int page_size;
+  int page_shift;  // log2(page_size), or -1 if it is not a power of two
   const int32_t *slot_epoch;  // (Hkv, p_len / page_size): epoch of a slot's last re-assignment
   int64_t slot_epoch_head_stride;
   const int32_t *epoch;       // the current epoch (one int32)
@@ -98,14 +173,16 @@ struct LocalLen {
 };
 __device__ __forceinline__ LocalLen local_len(const AttnArgs &a) {
   int64_t c_len = a.c_len;
-  if (a.c_len_dev) c_len = *a.c_len_dev;
+  if (a.c_len_dev) c_len += *a.c_len_dev;  // host value = offset to the device counter
   if (c_len < 0) c_len = 0;
   const bool has_new = a.new_k != nullptr && c_len < a.c_capacity;
   if (c_len > a.c_capacity) c_len = a.c_capacity;
   return {c_len, has_new};
 }
 
-template <typename T, int kLanes, int kRows>
+// kTail = false: chunks of the prefix and local segments; kTail = true: chunks
+// of the tail segment (the slots listed in the miss list).
+template <typename T, int kLanes, int kRows, bool kTail>
 __global__ void __launch_bounds__(kAttnThreads)
 decode_attention_split_kernel(const AttnArgs a) {
   constexpr int V = T::kVec;
@@ -121,7 +198,7 @@ decode_attention_split_kernel(const AttnArgs a) {
   const int chunk_id = a.chunk_base + blockIdx.x;
 
   // Which segment, which token range.
-  const int kind = chunk_id < a.n_pchunks ? 0 : (chunk_id < a.n_pchunks + a.n_lchunks ? 1 : 2);
+  const int kind = kTail ? 2 : (chunk_id < a.n_pchunks ? 0 : 1);
   const LocalLen ll = local_len(a);
   const int64_t c_len = ll.c_len;
   int64_t seg_len, t_begin;
@@ -133,10 +210,11 @@ decode_attention_split_kernel(const AttnArgs a) {
     t_begin = (int64_t)(chunk_id - a.n_pchunks) * a.chunk;
   } else {
     seg_len = (int64_t)a.miss_count[h] * a.page_size;
-    t_begin = (int64_t)(chunk_id - a.n_pchunks - a.n_lchunks) * a.chunk;
+    t_begin = (int64_t)(chunk_id - a.n_pchunks - a.n_lchunks) * a.tail_chunk;
   }
   if (t_begin >= seg_len) return;  // the merge kernel skips this chunk as well
-  const int64_t t_end = t_begin + a.chunk < seg_len ? t_begin + a.chunk : seg_len;
+  const int chunk = kind == 2 ? a.tail_chunk : a.chunk;
+  const int64_t t_end = t_begin + chunk < seg_len ? t_begin + chunk : seg_len;
 
   const char *kbase, *vbase;
   int64_t tok_stride_b;
@@ -158,6 +236,8 @@ decode_attention_split_kernel(const AttnArgs a) {
   const int32_t epoch_now = skip_fresh ? *a.epoch : 0;
   const int32_t *slot_epoch = skip_fresh ? a.slot_epoch + h * a.slot_epoch_head_stride : nullptr;
   const int32_t *miss_slot = kind == 2 ? a.miss_slot + (int64_t)h * a.miss_capacity : nullptr;
+  const bool uniform_pages = skip_fresh && a.page_shift >= 0 &&
+                             a.page_size % kStepTokens == 0 && a.chunk % a.page_size == 0;
 
   u32x4 qv[kRows];
 #pragma unroll
@@ -188,24 +268,28 @@ decode_attention_split_kernel(const AttnArgs a) {
       valid[u] = tok < t_end;
       int64_t tk = valid[u] ? tok : t_begin;  // clamp the address, mask the score
       if (skip_fresh) {
-        // a slot that is being rewritten right now is left to the tail pass
-        if (slot_epoch[tk / a.page_size] == epoch_now) valid[u] = false;
-      } else if (kind == 2) {
-        const int32_t slot = miss_slot[tk / a.page_size];
+        // A slot that is being rewritten right now is left to the tail pass; its
+        // rows are still loaded (no dependent address) and discarded below.  When
+        // a block step never straddles a page, the page is the same for the whole
+        // block and its epoch comes through the scalar cache.
+        int32_t ep;
+        if (uniform_pages)
+          ep = slot_epoch[(base + (int64_t)u * kStepTokens) >> a.page_shift];
+        else
+          ep = slot_epoch[a.page_shift >= 0 ? tk >> a.page_shift : tk / a.page_size];
+        if (ep == epoch_now) valid[u] = false;
+      } else if (kTail) {
+        const int64_t entry = a.page_shift >= 0 ? tk >> a.page_shift : tk / a.page_size;
+        const int64_t within = tk - entry * a.page_size;
+        const int32_t slot = miss_slot[entry];
         if (slot < 0) valid[u] = false;  // entry superseded later in the same step
-        tk = (int64_t)(slot < 0 ? 0 : slot) * a.page_size + tk % a.page_size;
+        tk = (int64_t)(slot < 0 ? 0 : slot) * a.page_size + within;
       }
       const bool is_new = newk != nullptr && tk == c_len;
       const char *kp = is_new ? newk : kbase + tk * tok_stride_b;
       const char *vp = is_new ? newv : vbase + tk * tok_stride_b;
-      if (skip_fresh && !valid[u]) {
-        // never touch memory another stream is writing: torn values could be NaN
-        kk[u] = u32x4{0, 0, 0, 0};
-        vv[u] = u32x4{0, 0, 0, 0};
-      } else {
-        kk[u] = load16(kp);
-        vv[u] = load16(vp);
-      }
+      kk[u] = load16(kp);
+      vv[u] = load16(vp);
       if (is_new && valid[u] && blockIdx.z == 0) {
         // the append: this lane group owns the new token's row
         store16(a.ck + (h * a.c_head_stride + c_len * a.c_tok_stride) * T::kBytes + c * 16, kk[u]);
@@ -213,19 +297,21 @@ decode_attention_split_kernel(const AttnArgs a) {
       }
     }
 #pragma unroll
-    for (int u = 0; u < kAttnUnroll; ++u) {
-      float s[kRows];
+    for (int u = 0; u < kAttnUnroll; u += 2) {
+      float s0[kRows], s1[kRows];
       bool grow = false;
 #pragma unroll
       for (int r = 0; r < kRows; ++r) {
-        s[r] = group_sum<kLanes>(dot16<T>(qv[r], kk[u])) * a.scale_log2;
-        if (!valid[u]) s[r] = -INFINITY;
-        grow |= s[r] > m[r];
+        s0[r] = group_sum<kLanes>(dot16<T>(qv[r], kk[u])) * a.scale_log2;
+        s1[r] = group_sum<kLanes>(dot16<T>(qv[r], kk[u + 1])) * a.scale_log2;
+        if (!valid[u]) s0[r] = -INFINITY;
+        if (!valid[u + 1]) s1[r] = -INFINITY;
+        grow |= fmaxf(s0[r], s1[r]) > m[r] + kRescaleSlack;
       }
-      if (__any(grow)) {  // rare after the first few tokens: rescale lazily
+      if (__any(grow)) {  // rare: the reference only moves when a score clears it by the slack
 #pragma unroll
         for (int r = 0; r < kRows; ++r) {
-          const float mn = fmaxf(m[r], s[r]);
+          const float mn = fmaxf(m[r], fmaxf(s0[r], s1[r]));
           const float alpha = fast_exp2(m[r] - mn);
           m[r] = mn;
           l[r] *= alpha;
@@ -233,15 +319,18 @@ decode_attention_split_kernel(const AttnArgs a) {
           for (int i = 0; i < V; ++i) acc[r][i] *= alpha;
         }
       }
-      float vf[V];
-      unpack<T>(vv[u], vf);
+      // a masked row may be memory another stream is writing (torn values, NaN):
+      // its weight is 0, and its values are zeroed so that 0 * NaN cannot arise
+      if (!valid[u]) vv[u] = u32x4{0, 0, 0, 0};
+      if (!valid[u + 1]) vv[u + 1] = u32x4{0, 0, 0, 0};
+      float p0[kRows], p1[kRows];
 #pragma unroll
       for (int r = 0; r < kRows; ++r) {
-        const float p = fast_exp2(s[r] - m[r]);
-        l[r] += p;
-#pragma unroll
-        for (int i = 0; i < V; ++i) acc[r][i] = fmaf(p, vf[i], acc[r][i]);
+        p0[r] = fast_exp2(s0[r] - m[r]);
+        p1[r] = fast_exp2(s1[r] - m[r]);
+        l[r] += p0[r] + p1[r];
       }
+      PvPair<T, kRows>::run(vv[u], vv[u + 1], p0, p1, acc);
     }
   }
 
@@ -309,6 +398,7 @@ decode_attention_split_kernel(const AttnArgs a) {
 // (at D = 128) chunk, reads the partial rows as 16-byte lanes, and the chunk
 // lanes are folded through LDS.
 constexpr int kMergeThreads = 512;
+constexpr int kMergeStats = 2048;  // (max, sum) pairs staged in LDS
 
 template <typename T>
 __global__ void __launch_bounds__(kMergeThreads)
@@ -324,7 +414,7 @@ decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__
   int n_t = 0;                                              // live tail chunks
   if (a.n_tchunks > 0) {
     const int64_t tail = (int64_t)a.miss_count[hq / a.rep] * a.page_size;
-    n_t = (int)((tail + a.chunk - 1) / a.chunk);
+    n_t = (int)((tail + a.tail_chunk - 1) / a.tail_chunk);
   }
   const int n_live = n_p + n_l + n_t;
   // i-th live chunk -> chunk id
@@ -332,15 +422,27 @@ decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__
     return i < n_p + n_l ? i : a.n_pchunks + a.n_lchunks + (i - n_p - n_l);
   };
 
+  // Stage the (max, sum) pairs of the live chunks in LDS with one load per
+  // thread, then let every wave reduce them for itself (no second barrier).
+  __shared__ float2 sm_ml[kMergeStats];
+  const bool staged = n_live <= kMergeStats;
+  if (staged) {
+    for (int i = t; i < n_live; i += kMergeThreads)
+      sm_ml[i] = *(const float2 *)(a.part_ml + ((int64_t)chunk_of(i) * a.n_q_heads + hq) * 2);
+    __syncthreads();
+  }
+  auto stat = [&](int i) -> float2 {
+    return staged ? sm_ml[i]
+                  : *(const float2 *)(a.part_ml + ((int64_t)chunk_of(i) * a.n_q_heads + hq) * 2);
+  };
   float mx = kMinusHuge;
-  for (int i = lane; i < n_live; i += 64)
-    mx = fmaxf(mx, a.part_ml[((int64_t)chunk_of(i) * a.n_q_heads + hq) * 2]);
+  for (int i = lane; i < n_live; i += 64) mx = fmaxf(mx, stat(i).x);
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
   float lt = 0.f;
   for (int i = lane; i < n_live; i += 64) {
-    const float *ml = a.part_ml + ((int64_t)chunk_of(i) * a.n_q_heads + hq) * 2;
-    lt += ml[1] * fast_exp2(ml[0] - mx);
+    const float2 ml = stat(i);
+    lt += ml.y * fast_exp2(ml.x - mx);
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) lt += __shfl_xor(lt, d, 64);
@@ -352,14 +454,25 @@ decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__
   const int qd = t % quads, cl = t / quads;
   float at[4] = {0.f, 0.f, 0.f, 0.f};
   if (cl < lanes_c) {
-    for (int i = cl; i < n_live; i += lanes_c) {
-      const int64_t slot = (int64_t)chunk_of(i) * a.n_q_heads + hq;
-      const float w = fast_exp2(a.part_ml[slot * 2] - mx);
-      const float4 v = *(const float4 *)(a.part_acc + slot * head_dim + qd * 4);
-      at[0] = fmaf(v.x, w, at[0]);
-      at[1] = fmaf(v.y, w, at[1]);
-      at[2] = fmaf(v.z, w, at[2]);
-      at[3] = fmaf(v.w, w, at[3]);
+    // four independent partial rows in flight per thread
+    for (int i0 = cl; i0 < n_live; i0 += 4 * lanes_c) {
+      float4 v[4];
+      float w[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * lanes_c;
+        const int ic = i < n_live ? i : cl;  // clamp the address, zero the weight
+        const int64_t slot = (int64_t)chunk_of(ic) * a.n_q_heads + hq;
+        v[u] = *(const float4 *)(a.part_acc + slot * head_dim + qd * 4);
+        w[u] = i < n_live ? fast_exp2(stat(ic).x - mx) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        at[0] = fmaf(v[u].x, w[u], at[0]);
+        at[1] = fmaf(v[u].y, w[u], at[1]);
+        at[2] = fmaf(v[u].z, w[u], at[2]);
+        at[3] = fmaf(v[u].w, w[u], at[3]);
+      }
     }
   }
 #pragma unroll
@@ -375,8 +488,12 @@ decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__
 }
 
 static int pick_chunk(int64_t total_tokens, int n_kv_heads, int step_tokens) {
-  // aim at ~8 blocks per CU on a 256-CU part, never below one unrolled round
-  const int64_t want_blocks = 256 * 8;
+  // ~8 blocks per CU on a 256-CU part (measured best on the 128K workload, alone
+  // and next to a running page stream); never below one unrolled round.
+  int64_t want_blocks = 256 * 8;
+#ifdef DA_TUNE
+  if (const char *e = getenv("DA_ATTN_BLOCKS")) want_blocks = atoi(e);
+#endif
   int64_t chunk = total_tokens * n_kv_heads / want_blocks;
   const int round = step_tokens * kAttnUnroll;
   if (chunk < round) chunk = round;
@@ -392,7 +509,7 @@ static int lanes_of(int head_dim, int dtype) {
 }
 
 struct ChunkPlan {
-  int chunk, n_p, n_l, n_t;
+  int chunk, tail_chunk, n_p, n_l, n_t;
   int64_t total() const { return (int64_t)n_p + n_l + n_t; }
 };
 // The chunk geometry of a launch; a function of the shapes only, so that the
@@ -404,7 +521,10 @@ static ChunkPlan plan_chunks(int n_kv_heads, int lanes, int64_t p_len, int64_t c
   p.chunk = pick_chunk(p_len + c_capacity, n_kv_heads, step_tokens);
   p.n_p = (int)ceil_div(p_len, p.chunk);
   p.n_l = (int)ceil_div(c_capacity, p.chunk);
-  p.n_t = (int)ceil_div(miss_tokens, p.chunk);
+  // the tail is short and every block starts with a dependent slot lookup:
+  // one unrolled round per block keeps it wide instead of deep
+  p.tail_chunk = step_tokens * kAttnUnroll;
+  p.n_t = (int)ceil_div(miss_tokens, p.tail_chunk);
   return p;
 }
 
@@ -412,21 +532,26 @@ static size_t attn_workspace_bytes(int n_q_heads, int head_dim, int64_t n_chunks
   return (size_t)n_chunks * n_q_heads * (head_dim + 2) * sizeof(float);
 }
 
-template <typename T, int kLanes>
+template <typename T, int kLanes, bool kTail>
 static void launch_split(AttnArgs a, int first_chunk, int n_launch, int n_kv_heads,
                          hipStream_t s) {
   if (n_launch <= 0) return;
   a.chunk_base = first_chunk;
   const int rep = a.rep;
   if (rep <= 1) {
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 1>),
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 1, kTail>),
                        dim3(n_launch, n_kv_heads, 1), dim3(kAttnThreads), 0, s, a);
   } else if (rep == 2) {
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 2>),
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 2, kTail>),
                        dim3(n_launch, n_kv_heads, 1), dim3(kAttnThreads), 0, s, a);
-  } else {
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 4>),
+  } else if (rep <= 4 || kLanes > 16) {
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 4, kTail>),
                        dim3(n_launch, n_kv_heads, (unsigned)ceil_div(rep, 4)),
+                       dim3(kAttnThreads), 0, s, a);
+  } else {
+    // eight query heads per kv head: keep all of them on one read of K/V
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, (kLanes > 16 ? 16 : kLanes), 8, kTail>),
+                       dim3(n_launch, n_kv_heads, (unsigned)ceil_div(rep, 8)),
                        dim3(kAttnThreads), 0, s, a);
   }
 }
@@ -435,22 +560,22 @@ static void launch_split(AttnArgs a, int first_chunk, int n_launch, int n_kv_hea
 template <typename T>
 static int launch_attention(const AttnArgs &a, int phase, int n_kv_heads, int lanes, int head_dim,
                             void *out, int64_t out_head_stride, float *lse_out, hipStream_t s) {
-#define DA_ATTN_LAUNCH(first, count)                                  \
-  switch (lanes) {                                                    \
-    case 4: launch_split<T, 4>(a, first, count, n_kv_heads, s); break;   \
-    case 8: launch_split<T, 8>(a, first, count, n_kv_heads, s); break;   \
-    case 16: launch_split<T, 16>(a, first, count, n_kv_heads, s); break; \
-    case 32: launch_split<T, 32>(a, first, count, n_kv_heads, s); break; \
-    case 64: launch_split<T, 64>(a, first, count, n_kv_heads, s); break; \
+#define DA_ATTN_LAUNCH(tail, first, count)                                     \
+  switch (lanes) {                                                             \
+    case 4: launch_split<T, 4, tail>(a, first, count, n_kv_heads, s); break;   \
+    case 8: launch_split<T, 8, tail>(a, first, count, n_kv_heads, s); break;   \
+    case 16: launch_split<T, 16, tail>(a, first, count, n_kv_heads, s); break; \
+    case 32: launch_split<T, 32, tail>(a, first, count, n_kv_heads, s); break; \
+    case 64: launch_split<T, 64, tail>(a, first, count, n_kv_heads, s); break; \
   }
   if (phase & 1) {
-    DA_ATTN_LAUNCH(0, a.n_pchunks + a.n_lchunks)
+    DA_ATTN_LAUNCH(false, 0, a.n_pchunks + a.n_lchunks)
     int rc = launch_status("da_decode_attention(split)");
     if (rc) return rc;
   }
   if (phase & 2) {
     if (a.n_tchunks > 0) {
-      DA_ATTN_LAUNCH(a.n_pchunks + a.n_lchunks, a.n_tchunks)
+      DA_ATTN_LAUNCH(true, a.n_pchunks + a.n_lchunks, a.n_tchunks)
       int rc = launch_status("da_decode_attention(tail)");
       if (rc) return rc;
     }
@@ -489,7 +614,8 @@ extern "C" int da_decode_attention_paged(
              n_kv_heads);
   DA_REQUIRE(dtype == DA_F32 || dtype == DA_F16 || dtype == DA_BF16,
              "da_decode_attention: unknown dtype %d", dtype);
-  DA_REQUIRE(p_len >= 0 && c_capacity >= 0 && c_len >= 0, "da_decode_attention: negative length");
+  DA_REQUIRE(p_len >= 0 && c_capacity >= 0 && (c_len >= 0 || c_len_dev),
+             "da_decode_attention: negative length");
   DA_REQUIRE(q && out && workspace, "da_decode_attention: null pointer");
   DA_REQUIRE(p_len == 0 || (pk && pv), "da_decode_attention: null prefix segment");
   DA_REQUIRE(c_capacity == 0 || (ck && cv), "da_decode_attention: null local cache");
@@ -548,6 +674,9 @@ extern "C" int da_decode_attention_paged(
     DA_REQUIRE(overlap->phase >= 1 && overlap->phase <= 3, "da_decode_attention: bad phase %d",
                overlap->phase);
     a.page_size = overlap->page_size;
+    a.page_shift = -1;
+    for (int b = 0; b < 31; ++b)
+      if ((1 << b) == overlap->page_size) a.page_shift = b;
     a.slot_epoch = overlap->slot_epoch;
     a.slot_epoch_head_stride = overlap->slot_epoch_head_stride;
     a.epoch = overlap->epoch;
@@ -559,6 +688,7 @@ extern "C" int da_decode_attention_paged(
   }
   const ChunkPlan p = plan_chunks(n_kv_heads, lanes, p_len, c_capacity, miss_tokens);
   a.chunk = p.chunk;
+  a.tail_chunk = p.tail_chunk;
   a.n_pchunks = p.n_p;
   a.n_lchunks = p.n_l;
   a.n_tchunks = p.n_t;

@@ -320,7 +320,7 @@ extern "C" int da_pages_gather(const void *dram, int64_t dram_head_stride_bytes,
                                int64_t hbm_head_stride_bytes, int64_t hbm_slot_stride_bytes,
                                int64_t page_bytes, const int32_t *miss_page,
                                const int32_t *miss_slot, const int32_t *miss_count,
-                               int n_kv_heads, int k, void *stream) {
+                               int n_kv_heads, int k, int max_blocks, void *stream) {
   using namespace da;
   DA_REQUIRE(n_kv_heads >= 0 && k >= 0 && page_bytes >= 0, "da_pages_gather: bad geometry");
   if (n_kv_heads == 0 || k == 0 || page_bytes == 0) return DA_OK;
@@ -333,7 +333,7 @@ extern "C" int da_pages_gather(const void *dram, int64_t dram_head_stride_bytes,
   DA_REQUIRE(n_kv_heads <= 65535, "da_pages_gather: too many heads");
   // Few, fat workgroups: ~32 blocks (16 KiB of reads in flight each) already
   // saturate the host link, and more concurrent page streams only lower it.
-  int cap = 32 / n_kv_heads;
+  int cap = (max_blocks > 0 ? max_blocks : 32) / n_kv_heads;
   if (cap < 1) cap = 1;
   const int per_head = k < cap ? k : cap;
   dim3 grid(per_head, n_kv_heads);

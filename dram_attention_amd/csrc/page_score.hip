@@ -12,6 +12,9 @@
 // keeps its slice of up to kRows query rows in registers, accumulates in fp32
 // and the kLanes partial sums are folded with wavefront shuffles.
 #include "common.hpp"
+#ifdef DA_TUNE
+#include <stdlib.h>
+#endif
 
 namespace da {
 
@@ -68,7 +71,7 @@ __global__ void __launch_bounds__(256)
 page_score_vec_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t q_head_stride,
                       const char *__restrict__ mm, int n_rows, int64_t n_pages,
                       OutT *__restrict__ out, int64_t out_row_stride, int64_t out_head_stride,
-                      int round_out) {
+                      int round_out, int rounds) {
   constexpr int V = T::kVec;
   constexpr int kGroups = 64 / kLanes;  // pages per wave step
   constexpr int kRowBytes = kLanes * 16;
@@ -87,10 +90,13 @@ page_score_vec_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t 
               qf[r]);
   }
 
-  const int64_t pages_per_block = (int64_t)(blockDim.x >> 6) * kGroups * kUnroll;
-  const int64_t p_first = blockIdx.x * pages_per_block + (int64_t)wave * kGroups * kUnroll;
+  const int64_t pages_per_round = (int64_t)(blockDim.x >> 6) * kGroups * kUnroll;
   const char *head_base = mm + (int64_t)h * n_pages * 2 * kRowBytes;
 
+  for (int round = 0; round < rounds; ++round) {
+  const int64_t p_first = ((int64_t)blockIdx.x * rounds + round) * pages_per_round +
+                          (int64_t)wave * kGroups * kUnroll;
+  if (p_first - (int64_t)wave * kGroups * kUnroll >= n_pages) break;
   u32x4 vmin[kUnroll], vmax[kUnroll];
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) {
@@ -124,6 +130,7 @@ page_score_vec_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t 
       }
     }
   }
+  }  // rounds
 }
 
 // Generic path: any head_dim, any strides.  One wave per page, lanes stride
@@ -159,19 +166,28 @@ static void launch_vec(const void *q, int64_t qrs, int64_t qhs, const void *mm, 
                        int n_heads, int64_t n_pages, OutT *out, int64_t ors, int64_t ohs,
                        int round_out, hipStream_t s) {
   constexpr int kGroups = 64 / kLanes;
+  // rounds per block: enough blocks to fill the part a few times over, but each
+  // block amortises its query load over several rounds of pages
+  int rounds = 1;
+#ifdef DA_TUNE
+  if (const char *e = getenv("DA_SCORE_ROUNDS")) rounds = atoi(e);
+#endif
   if (n_rows <= 4) {
-    constexpr int kRows = 4, kUnroll = 4;
-    dim3 grid((unsigned)ceil_div(n_pages, 4 * kGroups * kUnroll), n_heads, 1);
+#ifndef DA_SCORE_UNROLL
+#define DA_SCORE_UNROLL 2
+#endif
+    constexpr int kRows = 4, kUnroll = DA_SCORE_UNROLL;
+    dim3 grid((unsigned)ceil_div(n_pages, 4 * kGroups * kUnroll * rounds), n_heads, 1);
     hipLaunchKernelGGL((page_score_vec_kernel<T, kLanes, kRows, kUnroll, OutT>), grid, dim3(256),
                        0, s, (const char *)q, qrs, qhs, (const char *)mm, n_rows, n_pages, out,
-                       ors, ohs, round_out);
+                       ors, ohs, round_out, rounds);
   } else {
     constexpr int kRows = 8, kUnroll = 2;
-    dim3 grid((unsigned)ceil_div(n_pages, 4 * kGroups * kUnroll), n_heads,
+    dim3 grid((unsigned)ceil_div(n_pages, 4 * kGroups * kUnroll * rounds), n_heads,
               (unsigned)ceil_div(n_rows, kRows));
     hipLaunchKernelGGL((page_score_vec_kernel<T, kLanes, kRows, kUnroll, OutT>), grid, dim3(256),
                        0, s, (const char *)q, qrs, qhs, (const char *)mm, n_rows, n_pages, out,
-                       ors, ohs, round_out);
+                       ors, ohs, round_out, rounds);
   }
 }
 

@@ -66,12 +66,15 @@ def decode_attention(
     lse: torch.Tensor | None = None,
     scale: float | None = None,
     paged: PagedPrefix | None = None,
+    cache_len_offset: int = 0,
 ) -> torch.Tensor:
     """One query token against [prefix ++ cache rows 0..cache_len ++ new token].
 
     xq (Hq, D); prefix_k/v (Hkv, T, D) views with a dense last axis (T may be 0);
-    cache_k/v (capacity, Hkv, D); cache_len an int or a one-element int32 GPU
-    tensor; new_k/new_v (Hkv, D) are appended at row cache_len (or None).
+    cache_k/v (capacity, Hkv, D); cache_len an int, or a one-element int32 GPU
+    tensor to which ``cache_len_offset`` is added inside the kernel (so a device
+    position counter needs no arithmetic launch); new_k/new_v (Hkv, D) are
+    appended at row cache_len (or None).
     Returns (Hq, D) in xq.dtype; fills ``lse`` (Hq, fp32) when given.
     With ``paged`` the work is split around a concurrent page stream; the same
     workspace and ``out`` must be passed to both phases.
@@ -93,7 +96,7 @@ def decode_attention(
         _lib.require_gpu(cache_len, "cache_len")
         if cache_len.dtype != torch.int32:
             raise TypeError("a device-side cache length must be int32")
-        len_host, len_dev = 0, cache_len.data_ptr()
+        len_host, len_dev = int(cache_len_offset), cache_len.data_ptr()
     else:
         len_host, len_dev = int(cache_len), None
     if scale is None:
@@ -243,9 +246,11 @@ class DRAMAttention(torch.nn.Module):
         if seqlen != 1:
             raise RuntimeError("generate handles one token per call")
         if isinstance(start_pos, torch.Tensor):
-            cache_len = (start_pos - self.dram_kv_cache_size).to(torch.int32).reshape(1)
+            # the position stays on the device; the kernel subtracts the paged prefix
+            cache_len = start_pos if start_pos.dtype == torch.int32 else start_pos.to(torch.int32)
+            offset = -self.dram_kv_cache_size
         else:
-            cache_len = int(start_pos) - self.dram_kv_cache_size
+            cache_len, offset = int(start_pos) - self.dram_kv_cache_size, 0
         out = torch.empty(1, 1, Hq, D, dtype=xq.dtype, device=xq.device)
         lru = self.lru_cache
         if not isinstance(lru, LRUCache):
@@ -256,7 +261,7 @@ class DRAMAttention(torch.nn.Module):
                                                       xq.device)
             decode_attention(xq[0, 0], prefix_k, prefix_v, self.cache_k[0], self.cache_v[0],
                              cache_len, xk[0, 0], xv[0, 0], workspace=self._workspace,
-                             out=out[0, 0])
+                             out=out[0, 0], cache_len_offset=offset)
             return out
 
         idx = lru.select_(xq)
@@ -271,6 +276,7 @@ class DRAMAttention(torch.nn.Module):
         if not self.overlap_page_stream:
             lru.gather_(idx.shape[1])
             decode_attention(*args, workspace=self._workspace, out=out[0, 0],
+                             cache_len_offset=offset,
                              paged=PagedPrefix(self.page_size, scratch, lru.current_step, 3))
             return out
         main = torch.cuda.current_stream(xq.device)
@@ -280,9 +286,9 @@ class DRAMAttention(torch.nn.Module):
         side.wait_stream(main)                      # the miss list is ready
         with torch.cuda.stream(side):
             lru.gather_(idx.shape[1])
-        decode_attention(*args, workspace=self._workspace, out=out[0, 0],
+        decode_attention(*args, workspace=self._workspace, out=out[0, 0], cache_len_offset=offset,
                          paged=PagedPrefix(self.page_size, scratch, lru.current_step, 1))
         main.wait_stream(side)                      # the pages have landed
-        decode_attention(*args, workspace=self._workspace, out=out[0, 0],
+        decode_attention(*args, workspace=self._workspace, out=out[0, 0], cache_len_offset=offset,
                          paged=PagedPrefix(self.page_size, scratch, lru.current_step, 2))
         return out

@@ -99,7 +99,7 @@ def lru_update(
 
 
 def pages_gather(dram_kv_cache: torch.Tensor, hbm_kv_cache: torch.Tensor, scratch: LruScratch,
-                 k: int, dram_device_ptr: Optional[int] = None) -> None:
+                 k: int, dram_device_ptr: Optional[int] = None, max_blocks: int = 0) -> None:
     """The data half: copy every page of the miss list into its slot (one launch
     on the current stream; the page store may be pinned host memory)."""
     num_heads, _, page_dim = dram_kv_cache.shape
@@ -112,7 +112,8 @@ def pages_gather(dram_kv_cache: torch.Tensor, hbm_kv_cache: torch.Tensor, scratc
             dram_device_ptr, dram_kv_cache.stride(0) * esz, dram_kv_cache.stride(1) * esz,
             hbm_kv_cache.data_ptr(), hbm_kv_cache.stride(0) * esz, hbm_kv_cache.stride(1) * esz,
             page_dim * esz, scratch.miss_page.data_ptr(), scratch.miss_slot.data_ptr(),
-            scratch.miss_count.data_ptr(), num_heads, k, _lib.stream_ptr(hbm_kv_cache.device),
+            scratch.miss_count.data_ptr(), num_heads, k, max_blocks,
+            _lib.stream_ptr(hbm_kv_cache.device),
         ),
         "da_pages_gather",
     )

@@ -153,14 +153,16 @@ int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_itype,
  *   dram : device-visible base of the (Hkv, P, page_bytes) page store
  *   hbm  : base of the (Hkv, N_hbm, page_bytes) slot array
  * Entry i < miss_count[h] of head h copies page miss_page[h,i] to slot
- * miss_slot[h,i]; page_bytes must be a multiple of 16.
+ * miss_slot[h,i]; page_bytes must be a multiple of 16.  max_blocks bounds the
+ * number of workgroups (0 = the default, 32: a few fat workgroups saturate the
+ * host link, more concurrent page streams only lower its throughput).
  */
 int da_pages_gather(const void *dram, int64_t dram_head_stride_bytes,
                     int64_t dram_page_stride_bytes, void *hbm,
                     int64_t hbm_head_stride_bytes, int64_t hbm_slot_stride_bytes,
                     int64_t page_bytes, const int32_t *miss_page,
                     const int32_t *miss_slot, const int32_t *miss_count,
-                    int n_kv_heads, int k, void *stream);
+                    int n_kv_heads, int k, int max_blocks, void *stream);
 
 /*
  * Subsystem 5 — split-K decode attention for ONE query token over
@@ -174,7 +176,8 @@ int da_pages_gather(const void *dram, int64_t dram_head_stride_bytes,
  *                  (p_head_stride, p_tok_stride, 1); p_len may be 0
  *   ck, cv       : local cache, (capacity, Hkv, D) addressed with (c_tok_stride, c_head_stride, 1)
  *   c_len        : rows already valid in the local cache; if c_len_dev is not
- *                  NULL the value is read from that device int32 instead
+ *                  NULL the count is *c_len_dev + c_len (a device position
+ *                  counter plus a host offset, which may be negative)
  *   new_k, new_v : (Hkv, D) of the current token (head stride new_head_stride),
  *                  or NULL to attend over the c_len cached rows only
  *   out          : (Hq, D) in `dtype`;  lse_out : optional (Hq) fp32, natural log

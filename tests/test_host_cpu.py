@@ -48,7 +48,7 @@ def test_argument_checks_reject_before_any_launch(lib):
     assert b"exceeds" in lib.da_last_error_string()
     assert lib.da_pages_gather(ctypes.c_void_p(16), 0, 0, ctypes.c_void_p(16), 0, 0, 24,
                                ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16),
-                               1, 1, None) == -1
+                               1, 1, 0, None) == -1
 
 
 def test_module_surface_and_errors_on_cpu():
