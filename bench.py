@@ -286,6 +286,10 @@ def main():
     score_gbps = (score_b / (kernel_us["page_score"] * 1e-6) / 1e9
                   if "page_score" in kernel_us else None)
 
+    # HBM bytes per launch of the roofline kernel from the committed counter runs
+    # (profiles/bench_128k_hbm_traffic_pmc.md: FETCH_SIZE x 2.0 + WRITE_SIZE); only
+    # known for the workload those runs used
+    traffic = 154.7e6 if w.name == "128k" else None
     result = {
         "metric": "decode steps/sec per layer at 128K ctx; scorer+attn HBM GB/s vs peak",
         "value": args.steps / dt,
@@ -311,7 +315,7 @@ def main():
         "roofline": {
             "bound": "hbm", "kernel": "decode_attention_split_kernel (prefix + local segments)",
             "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
             "algorithmic_bytes": attn_b, "avg_us": attn_us,
         },
         "kernels_us": kernel_us,
