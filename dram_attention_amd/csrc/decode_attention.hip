@@ -194,7 +194,8 @@ decode_attention_split_kernel(const AttnArgs a) {
   const int c = lane % kLanes;
   const int g = lane / kLanes;
   const int h = blockIdx.y;
-  const int row0 = blockIdx.z * kRows;  // first query row of the GQA group handled here
+  const int row_group = blockIdx.z;
+  const int row0 = row_group * kRows;  // first query row of the GQA group handled here
   const int chunk_id = a.chunk_base + blockIdx.x;
 
   // Which segment, which token range.
@@ -236,8 +237,19 @@ decode_attention_split_kernel(const AttnArgs a) {
   const int32_t epoch_now = skip_fresh ? *a.epoch : 0;
   const int32_t *slot_epoch = skip_fresh ? a.slot_epoch + h * a.slot_epoch_head_stride : nullptr;
   const int32_t *miss_slot = kind == 2 ? a.miss_slot + (int64_t)h * a.miss_capacity : nullptr;
+  // When a block step never straddles a page and the chunk has at most 64
+  // pages, one load per wave fetches the chunk's epochs and a ballot turns them
+  // into a bit mask: the token loop then needs no memory access for the test.
   const bool uniform_pages = skip_fresh && a.page_shift >= 0 &&
-                             a.page_size % kStepTokens == 0 && a.chunk % a.page_size == 0;
+                             a.page_size % kStepTokens == 0 && a.chunk % a.page_size == 0 &&
+                             (a.chunk >> a.page_shift) <= 64;
+  uint64_t fresh_mask = 0;
+  if (uniform_pages) {
+    const int64_t first_page = t_begin >> a.page_shift;
+    const int64_t n_pages_here = (t_end - t_begin + a.page_size - 1) >> a.page_shift;
+    const bool fresh = lane < n_pages_here && slot_epoch[first_page + lane] == epoch_now;
+    fresh_mask = __ballot(fresh);
+  }
 
   u32x4 qv[kRows];
 #pragma unroll
@@ -269,15 +281,13 @@ decode_attention_split_kernel(const AttnArgs a) {
       int64_t tk = valid[u] ? tok : t_begin;  // clamp the address, mask the score
       if (skip_fresh) {
         // A slot that is being rewritten right now is left to the tail pass; its
-        // rows are still loaded (no dependent address) and discarded below.  When
-        // a block step never straddles a page, the page is the same for the whole
-        // block and its epoch comes through the scalar cache.
-        int32_t ep;
+        // rows are still loaded (no dependent address) and discarded below.
+        bool fresh;
         if (uniform_pages)
-          ep = slot_epoch[(base + (int64_t)u * kStepTokens) >> a.page_shift];
+          fresh = (fresh_mask >> ((base - t_begin + (int64_t)u * kStepTokens) >> a.page_shift)) & 1;
         else
-          ep = slot_epoch[a.page_shift >= 0 ? tk >> a.page_shift : tk / a.page_size];
-        if (ep == epoch_now) valid[u] = false;
+          fresh = slot_epoch[a.page_shift >= 0 ? tk >> a.page_shift : tk / a.page_size] == epoch_now;
+        if (fresh) valid[u] = false;
       } else if (kTail) {
         const int64_t entry = a.page_shift >= 0 ? tk >> a.page_shift : tk / a.page_size;
         const int64_t within = tk - entry * a.page_size;
@@ -290,7 +300,7 @@ decode_attention_split_kernel(const AttnArgs a) {
       const char *vp = is_new ? newv : vbase + tk * tok_stride_b;
       kk[u] = load16(kp);
       vv[u] = load16(vp);
-      if (is_new && valid[u] && blockIdx.z == 0) {
+      if (is_new && valid[u] && row_group == 0) {
         // the append: this lane group owns the new token's row
         store16(a.ck + (h * a.c_head_stride + c_len * a.c_tok_stride) * T::kBytes + c * 16, kk[u]);
         store16(a.cv + (h * a.c_head_stride + c_len * a.c_tok_stride) * T::kBytes + c * 16, vv[u]);
@@ -488,9 +498,11 @@ decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__
 }
 
 static int pick_chunk(int64_t total_tokens, int n_kv_heads, int step_tokens) {
-  // ~8 blocks per CU on a 256-CU part (measured best on the 128K workload, alone
-  // and next to a running page stream); never below one unrolled round.
-  int64_t want_blocks = 256 * 8;
+  // ~2 blocks per CU on a 256-CU part: every block pays a fixed prologue and a
+  // merge epilogue, so few long chunks beat many short ones (measured on the
+  // 128K workload: 31.9 us at 512 blocks, 32.6 us at 2048); never below one
+  // unrolled round.
+  int64_t want_blocks = 256 * 2;
 #ifdef DA_TUNE
   if (const char *e = getenv("DA_ATTN_BLOCKS")) want_blocks = atoi(e);
 #endif
@@ -538,22 +550,19 @@ static void launch_split(AttnArgs a, int first_chunk, int n_launch, int n_kv_hea
   if (n_launch <= 0) return;
   a.chunk_base = first_chunk;
   const int rep = a.rep;
-  if (rep <= 1) {
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 1, kTail>),
-                       dim3(n_launch, n_kv_heads, 1), dim3(kAttnThreads), 0, s, a);
-  } else if (rep == 2) {
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 2, kTail>),
-                       dim3(n_launch, n_kv_heads, 1), dim3(kAttnThreads), 0, s, a);
-  } else if (rep <= 4 || kLanes > 16) {
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 4, kTail>),
-                       dim3(n_launch, n_kv_heads, (unsigned)ceil_div(rep, 4)),
+  // at most 4 query rows per block (8 would need all 256 vector registers and
+  // run at one wave per SIMD); larger GQA groups take several blocks per chunk
+  const int rows = rep <= 1 ? 1 : (rep == 2 ? 2 : 4);
+  const dim3 grid(n_launch, n_kv_heads, (unsigned)ceil_div(rep, rows));
+  if (rows == 1)
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 1, kTail>), grid,
                        dim3(kAttnThreads), 0, s, a);
-  } else {
-    // eight query heads per kv head: keep all of them on one read of K/V
-    hipLaunchKernelGGL((decode_attention_split_kernel<T, (kLanes > 16 ? 16 : kLanes), 8, kTail>),
-                       dim3(n_launch, n_kv_heads, (unsigned)ceil_div(rep, 8)),
+  else if (rows == 2)
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 2, kTail>), grid,
                        dim3(kAttnThreads), 0, s, a);
-  }
+  else
+    hipLaunchKernelGGL((decode_attention_split_kernel<T, kLanes, 4, kTail>), grid,
+                       dim3(kAttnThreads), 0, s, a);
 }
 
 // phase bit 1: prefix (minus fresh slots) + local segment; bit 2: tail + merge.
