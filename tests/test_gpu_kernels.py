@@ -282,7 +282,7 @@ def dense_reference(q, segments):
 @pytest.mark.parametrize("Hq,Hkv,D,p_len,c_len,cap", [
     (32, 8, 128, 2048, 500, 640), (8, 2, 64, 512, 1008, 1040), (4, 4, 128, 0, 77, 128),
     (16, 2, 64, 333, 0, 64), (6, 2, 128, 1000, 31, 32), (2, 1, 256, 40, 3, 8),
-    (64, 8, 128, 4096, 100, 200)])
+    (64, 8, 128, 4096, 100, 200), (12, 2, 128, 700, 45, 64), (32, 2, 64, 300, 9, 16)])
 def test_decode_attention_matches_dense(dtype, atol, rtol, Hq, Hkv, D, p_len, c_len, cap):
     from dram_attention_amd import decode_attention
 

@@ -243,6 +243,61 @@ def test_page_stream_overlap_changes_nothing():
         assert close(plain, b[0, 0], 1e-2, 1e-2)
 
 
+def test_graph_replay_equals_eager_steps():
+    """The whole step (selection, LRU, page stream on its side stream, two-phase
+    attention, append) captured once and replayed: every replay, with eager work
+    and synchronisations in between, gives the eager module's bits and state."""
+    from dram_attention_amd import DRAMAttention
+
+    w = WORKLOADS["128k"].scaled(dram_tokens=16384, local_cache=1024, lru_tokens=4096,
+                                 top_k_tokens=1024, steps=7)
+    prompt = make_prompt(w, 6)
+    mods = []
+    for _ in range(2):
+        m = DRAMAttention(w.steps + 1, w.lru_tokens, w.local_cache, 16, w.top_k_tokens, w.n_kv_heads,
+                          w.head_dim, device=DEV, dtype=w.dtype)
+        m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+        mods.append(m)
+    graphed, eager = mods
+    inputs = DecodeInputs(w, prompt.q0, 6)
+    steps = [tuple(x.to(DEV) for x in inputs.next()) for _ in range(w.steps)]
+    xq, xk, xv = (torch.empty_like(x) for x in steps[0])
+    pos = torch.tensor([w.prompt_tokens], dtype=torch.int32, device=DEV)
+
+    def feed(t):
+        for dst, src in zip((xq, xk, xv), steps[t]):
+            dst.copy_(src)
+
+    # step 0 eagerly on both (resolves the pinned mapping, sizes the workspaces)
+    feed(0)
+    a = graphed(xq, xk, xv, start_pos=pos, stage="generate")
+    b = eager(*steps[0], start_pos=w.prompt_tokens, stage="generate")
+    assert same(a, b)
+    pos += 1
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    feed(1)
+    with torch.cuda.graph(g):
+        out = graphed(xq, xk, xv, start_pos=pos, stage="generate")
+        pos += 1
+    # capture executes nothing, so the counters still stand at step 1
+    for t in range(1, w.steps):
+        feed(t)
+        g.replay()
+        want = eager(*steps[t], start_pos=w.prompt_tokens + t, stage="generate")
+        torch.cuda.synchronize()
+        assert pos.item() == w.prompt_tokens + t + 1
+        assert same(out, want), f"step {t}"
+        la, lb = graphed.lru_cache, eager.lru_cache
+        assert same(la.hbm_kv_cache, lb.hbm_kv_cache), f"slots, step {t}"
+        assert same(la.page_access_time, lb.page_access_time)
+        assert same(la.dram_page_to_hbm_page_mapping, lb.dram_page_to_hbm_page_mapping)
+        assert la.current_step.item() == lb.current_step.item() == t + 1
+        assert la.last_miss_counts().sum().item() > 0
+    c = w.prompt_tokens + w.steps - w.dram_tokens
+    assert same(graphed.cache_k[0, :c], eager.cache_k[0, :c])
+
+
 def test_static_prefix_equals_full_attention():
     """Prefix within the HBM budget: the static cache path is dense attention over
     the whole sequence (the 32K configuration through init_cache)."""
