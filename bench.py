@@ -115,7 +115,7 @@ def time_kernels(layer, steps):
 
     m, lru, w = layer.m, layer.m.lru_cache, layer.w
     names = ("page_score", "topk_pages", "lru_update", "pages_gather", "decode_attention_split",
-             "decode_attention_tail+merge")
+             "decode_attention_first_merge", "decode_attention_tail+merge")
     acc = {n: 0.0 for n in names}
     misses, local_rows = 0, []
     if not isinstance(lru, LRUCache):
@@ -166,12 +166,12 @@ def time_kernels(layer, steps):
         c_len = int(layer.pos_dev.item()) - m.dram_kv_cache_size
         args = (xq[0, 0], pk, pv, m.cache_k[0], m.cache_v[0], c_len, xk[0, 0], xv[0, 0])
         out = torch.empty(w.n_q_heads, w.head_dim, dtype=w.dtype, device=xq.device)
-        timed("decode_attention_split", lambda: decode_attention(
-            *args, workspace=m._workspace, out=out,
-            paged=PagedPrefix(w.page_size, scratch, lru.current_step, 1)))
-        timed("decode_attention_tail+merge", lambda: decode_attention(
-            *args, workspace=m._workspace, out=out,
-            paged=PagedPrefix(w.page_size, scratch, lru.current_step, 2)))
+        for name, phase in (("decode_attention_split", PagedPrefix.FIRST),
+                            ("decode_attention_first_merge", PagedPrefix.FIRST_MERGE),
+                            ("decode_attention_tail+merge", PagedPrefix.SECOND)):
+            timed(name, lambda phase=phase: decode_attention(
+                *args, workspace=m._workspace, out=out,
+                paged=PagedPrefix(w.page_size, scratch, lru.current_step, phase)))
         torch.cuda.synchronize()
         for name, e0, e1, repeat in pending:
             acc[name] += e0.elapsed_time(e1) / repeat

@@ -153,6 +153,7 @@ struct AttnArgs {
   // chunk ids: [0, n_pchunks) prefix, [n_pchunks, +n_lchunks) local, then n_tchunks tail
   int n_pchunks, n_lchunks, n_tchunks;
   int chunk_base;  // chunk id of blockIdx.x == 0 in this launch
+  int pre_chunk;   // chunk id that holds the merged result of the prefix and local chunks
   int n_q_heads;
   float *part_ml;   // (chunks, Hq, 2): running max (log2 domain), sum
   float *part_acc;  // (chunks, Hq, D)
@@ -408,12 +409,17 @@ decode_attention_split_kernel(const AttnArgs a) {
 // barrier); then a thread owns four adjacent output channels of every 16th
 // (at D = 128) chunk, reads the partial rows as 16-byte lanes, and the chunk
 // lanes are folded through LDS.
+//   kMergeAll   : every live chunk -> out
+//   kMergePre   : prefix and local chunks -> out, and their merged, unnormalised
+//                 state -> chunk `pre_chunk` (runs next to the page stream)
+//   kMergeFinal : chunk `pre_chunk` + the live tail chunks -> out
 constexpr int kMergeThreads = 512;
 constexpr int kMergeStats = 2048;  // (max, sum) pairs staged in LDS
+enum MergeMode { kMergeAll = 0, kMergePre = 1, kMergeFinal = 2 };
 
 template <typename T>
 __global__ void __launch_bounds__(kMergeThreads)
-decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__ out,
+decode_attention_merge_kernel(const AttnArgs a, int mode, int head_dim, char *__restrict__ out,
                               int64_t out_head_stride, float *__restrict__ lse_out) {
   const int hq = blockIdx.x;
   const int t = threadIdx.x;
@@ -423,14 +429,16 @@ decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__
   const int n_p = a.n_pchunks;                              // live prefix chunks (all of them)
   const int n_l = (int)((l_len + a.chunk - 1) / a.chunk);   // live local chunks
   int n_t = 0;                                              // live tail chunks
-  if (a.n_tchunks > 0) {
+  if (a.n_tchunks > 0 && mode != kMergePre) {
     const int64_t tail = (int64_t)a.miss_count[hq / a.rep] * a.page_size;
     n_t = (int)((tail + a.tail_chunk - 1) / a.tail_chunk);
   }
-  const int n_live = n_p + n_l + n_t;
+  const int n_first = mode == kMergeFinal ? 1 : n_p + n_l;  // chunks ahead of the tail's
+  const int n_live = n_first + n_t;
   // i-th live chunk -> chunk id
   auto chunk_of = [&](int i) {
-    return i < n_p + n_l ? i : a.n_pchunks + a.n_lchunks + (i - n_p - n_l);
+    if (i < n_first) return mode == kMergeFinal ? a.pre_chunk : i;
+    return a.n_pchunks + a.n_lchunks + (i - n_first);
   };
 
   // Stage the (max, sum) pairs of the live chunks in LDS with one load per
@@ -489,10 +497,16 @@ decode_attention_merge_kernel(const AttnArgs a, int head_dim, char *__restrict__
 #pragma unroll
   for (int i = 0; i < 4; ++i) sm_acc[t * 4 + i] = at[i];
   __syncthreads();
+  const int64_t pre_slot = (int64_t)a.pre_chunk * a.n_q_heads + hq;
   for (int d = t; d < head_dim; d += kMergeThreads) {
     float s = 0.f;
     for (int c2 = 0; c2 < lanes_c; ++c2) s += sm_acc[(c2 * quads + d / 4) * 4 + (d & 3)];
     store_elem<T>(out, (int64_t)hq * out_head_stride + d, s * inv);
+    if (mode == kMergePre) a.part_acc[pre_slot * head_dim + d] = s;
+  }
+  if (mode == kMergePre && t == 0) {
+    a.part_ml[pre_slot * 2] = mx;
+    a.part_ml[pre_slot * 2 + 1] = lt;
   }
   if (lse_out && t == 0)
     lse_out[hq] = lt > 0.f ? (mx + __builtin_amdgcn_logf(lt)) * kLn2 : -INFINITY;
@@ -523,7 +537,9 @@ static int lanes_of(int head_dim, int dtype) {
 
 struct ChunkPlan {
   int chunk, tail_chunk, n_p, n_l, n_t;
-  int64_t total() const { return (int64_t)n_p + n_l + n_t; }
+  // one more slot than there are chunks: the merged state of the first pass
+  int64_t total() const { return (int64_t)n_p + n_l + n_t + 1; }
+  int pre_chunk() const { return n_p + n_l + n_t; }
 };
 // The chunk geometry of a launch; a function of the shapes only, so that the
 // workspace query and every phase of a step agree on it.
@@ -572,7 +588,10 @@ static void launch_split(AttnArgs a, int first_chunk, int n_launch, int n_kv_hea
                        dim3(kAttnThreads), 0, s, a);
 }
 
-// phase bit 1: prefix (minus fresh slots) + local segment; bit 2: tail + merge.
+// DA_PHASE_FIRST: prefix (minus fresh slots) + local segment; DA_PHASE_SECOND: tail +
+// merge.  Issued as two calls around a page stream, the first call also merges its own
+// chunks (into `out` and into one partial), so that the second call, the part
+// the step waits for, merges only that partial and the tail's.
 template <typename T>
 static int launch_attention(const AttnArgs &a, int phase, int n_kv_heads, int lanes, int head_dim,
                             void *out, int64_t out_head_stride, float *lse_out, hipStream_t s) {
@@ -584,21 +603,33 @@ static int launch_attention(const AttnArgs &a, int phase, int n_kv_heads, int la
     case 32: launch_split<T, 32, tail>(a, first, count, n_kv_heads, s); break; \
     case 64: launch_split<T, 64, tail>(a, first, count, n_kv_heads, s); break; \
   }
-  if (phase & 1) {
+#define DA_ATTN_MERGE(mode)                                                                    \
+  hipLaunchKernelGGL(decode_attention_merge_kernel<T>, dim3(a.n_q_heads), dim3(kMergeThreads), \
+                     0, s, a, mode, head_dim, (char *)out, out_head_stride, lse_out)
+  if (phase & DA_PHASE_FIRST) {
     DA_ATTN_LAUNCH(false, 0, a.n_pchunks + a.n_lchunks)
     int rc = launch_status("da_decode_attention(split)");
     if (rc) return rc;
   }
-  if (phase & 2) {
+  if (phase & DA_PHASE_FIRST_MERGE) {
+    DA_ATTN_MERGE(kMergePre);
+    int rc = launch_status("da_decode_attention(merge of the first pass)");
+    if (rc) return rc;
+  }
+  if (phase & DA_PHASE_SECOND) {
+    // everything in one call and no carried partial: one merge over all chunks
+    const bool all = (phase & DA_PHASE_FIRST) && !(phase & DA_PHASE_FIRST_MERGE);
     if (a.n_tchunks > 0) {
       DA_ATTN_LAUNCH(true, a.n_pchunks + a.n_lchunks, a.n_tchunks)
       int rc = launch_status("da_decode_attention(tail)");
       if (rc) return rc;
+    } else if (!all) {
+      return DA_OK;  // the merge of the first pass already wrote the output
     }
-    hipLaunchKernelGGL(decode_attention_merge_kernel<T>, dim3(a.n_q_heads), dim3(kMergeThreads), 0,
-                       s, a, head_dim, (char *)out, out_head_stride, lse_out);
+    DA_ATTN_MERGE(all ? kMergeAll : kMergeFinal);
     return launch_status("da_decode_attention(merge)");
   }
+#undef DA_ATTN_MERGE
 #undef DA_ATTN_LAUNCH
   return DA_OK;
 }
@@ -687,7 +718,7 @@ extern "C" int da_decode_attention_paged(
     DA_REQUIRE(overlap->slot_epoch && overlap->epoch && overlap->miss_slot &&
                    overlap->miss_count && overlap->miss_capacity >= 0,
                "da_decode_attention: incomplete overlap description");
-    DA_REQUIRE(overlap->phase >= 1 && overlap->phase <= 3, "da_decode_attention: bad phase %d",
+    DA_REQUIRE(overlap->phase >= 1 && overlap->phase <= 7, "da_decode_attention: bad phase %d",
                overlap->phase);
     a.page_size = overlap->page_size;
     a.page_shift = -1;
@@ -708,6 +739,7 @@ extern "C" int da_decode_attention_paged(
   a.n_pchunks = p.n_p;
   a.n_lchunks = p.n_l;
   a.n_tchunks = p.n_t;
+  a.pre_chunk = p.pre_chunk();
   const size_t need = attn_workspace_bytes(n_q_heads, head_dim, p.total());
   DA_REQUIRE(workspace_bytes >= need, "da_decode_attention: workspace %zu < %zu bytes",
              workspace_bytes, need);

@@ -23,9 +23,12 @@ class PagedPrefix:
     """Says that the prefix handed to :func:`decode_attention` is the slot array of
     an LRU page cache whose page stream for this step may still be running.
 
-    phase 1 attends over the local window and every slot that keeps its page,
-    phase 2 (after the stream has finished) over the re-assigned slots and writes
-    the output, phase 3 does both at once."""
+    FIRST attends over the local window and every slot that keeps its page,
+    FIRST_MERGE folds those partial results into one (both may run next to the
+    stream), SECOND (after the stream has finished) attends over the re-assigned
+    slots and writes the output; FIRST | SECOND does everything at once."""
+
+    FIRST, SECOND, FIRST_MERGE = 1, 2, 4
 
     def __init__(self, page_size: int, scratch, current_step: torch.Tensor, phase: int):
         self.page_size = page_size
@@ -77,7 +80,7 @@ def decode_attention(
     appended at row cache_len (or None).
     Returns (Hq, D) in xq.dtype; fills ``lse`` (Hq, fp32) when given.
     With ``paged`` the work is split around a concurrent page stream; the same
-    workspace and ``out`` must be passed to both phases.
+    workspace and ``out`` must be passed to every call of the step.
     """
     Hq, D = xq.shape
     Hkv = cache_k.shape[1]
@@ -277,7 +280,10 @@ class DRAMAttention(torch.nn.Module):
             lru.gather_(idx.shape[1])
             decode_attention(*args, workspace=self._workspace, out=out[0, 0],
                              cache_len_offset=offset,
-                             paged=PagedPrefix(self.page_size, scratch, lru.current_step, 3))
+                             # the same kernels as the overlapped order, so the same bits
+                             paged=PagedPrefix(self.page_size, scratch, lru.current_step,
+                                               PagedPrefix.FIRST | PagedPrefix.FIRST_MERGE |
+                                               PagedPrefix.SECOND))
             return out
         main = torch.cuda.current_stream(xq.device)
         if self._side_stream is None:
@@ -287,8 +293,10 @@ class DRAMAttention(torch.nn.Module):
         with torch.cuda.stream(side):
             lru.gather_(idx.shape[1])
         decode_attention(*args, workspace=self._workspace, out=out[0, 0], cache_len_offset=offset,
-                         paged=PagedPrefix(self.page_size, scratch, lru.current_step, 1))
+                         paged=PagedPrefix(self.page_size, scratch, lru.current_step,
+                                           PagedPrefix.FIRST | PagedPrefix.FIRST_MERGE))
         main.wait_stream(side)                      # the pages have landed
         decode_attention(*args, workspace=self._workspace, out=out[0, 0], cache_len_offset=offset,
-                         paged=PagedPrefix(self.page_size, scratch, lru.current_step, 2))
+                         paged=PagedPrefix(self.page_size, scratch, lru.current_step,
+                                           PagedPrefix.SECOND))
         return out

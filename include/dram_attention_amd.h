@@ -204,18 +204,33 @@ int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
  * and the missed pages of this step are streamed in concurrently on another
  * stream (no counterpart in the reference, whose page copies and attention are
  * serialised on one stream, dram_attention/dram_attention.py:161-172).
- *   phase 1 : local segment + every slot whose slot_epoch differs from *epoch;
- *             may run while da_pages_gather is still writing the other slots
- *   phase 2 : the slots listed in miss_slot[h, 0..miss_count[h]) (entries of -1
- *             are skipped), then the merge that writes `out`; issue it after the
- *             page stream has completed
- *   phase 3 : both, back to back (the page stream must have completed)
- * The two phases of a step must be given identical arguments otherwise.  The
+ * `phase` is a set of DA_PHASE_* bits, carried out in this order:
+ *   DA_PHASE_FIRST       : local segment + every slot whose slot_epoch differs
+ *                          from *epoch; may run while da_pages_gather is still
+ *                          writing the other slots
+ *   DA_PHASE_FIRST_MERGE : merges the partial results of DA_PHASE_FIRST into one
+ *                          partial kept in the workspace, and into `out` (the
+ *                          result without the slots the second pass covers);
+ *                          may also run next to the page stream
+ *   DA_PHASE_SECOND      : the slots listed in miss_slot[h, 0..miss_count[h])
+ *                          (entries of -1 are skipped), then the merge that
+ *                          writes the complete `out` and `lse_out`; issue it
+ *                          after the page stream has completed.  Without
+ *                          DA_PHASE_FIRST in the same call it merges the tail with
+ *                          the partial DA_PHASE_FIRST_MERGE left in the workspace.
+ * The usual step: FIRST | FIRST_MERGE next to the stream, SECOND after the join.
+ * FIRST | SECOND in one call (the page stream already complete) needs no
+ * FIRST_MERGE.
+ * The calls of a step must be given identical arguments otherwise.  The
  * workspace needs miss_tokens = miss_capacity * page_size.
  */
+#define DA_PHASE_FIRST 1
+#define DA_PHASE_SECOND 2
+#define DA_PHASE_FIRST_MERGE 4
+
 typedef struct da_paged_overlap {
   int32_t page_size;              /* tokens per slot; p_len = slots * page_size */
-  int32_t phase;                  /* 1, 2 or 3 */
+  int32_t phase;                  /* DA_PHASE_* bits */
   const int32_t *slot_epoch;      /* (Hkv, slots), written by da_lru_update */
   int64_t slot_epoch_head_stride; /* elements */
   const int32_t *epoch;           /* the LRU step counter after da_lru_update */
