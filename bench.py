@@ -20,6 +20,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -110,6 +111,7 @@ def time_kernels(layer, steps):
     stream runs to completion before attention here (no overlap), so each kernel
     is seen alone."""
     from dram_attention_amd.dram_attention import PagedPrefix, decode_attention
+    from dram_attention_amd.lru_kernel import GATHER_BLOCKS, gather_attend_supported
 
     from dram_attention_amd import LRUCache
 
@@ -161,17 +163,25 @@ def time_kernels(layer, steps):
         idx = lru._topk_idx
         timed("topk_pages", lambda: topk_pages(scores, w.rep, k, idx, w.rep * k, idx.shape[1], k))
         scratch = timed("lru_update", lambda: lru.update_(idx), repeat=1)   # mutates its state
-        timed("pages_gather", lambda: lru.gather_(idx.shape[1]))
         pk, pv = lru.views()
         c_len = int(layer.pos_dev.item()) - m.dram_kv_cache_size
         args = (xq[0, 0], pk, pv, m.cache_k[0], m.cache_v[0], c_len, xk[0, 0], xv[0, 0])
         out = torch.empty(w.n_q_heads, w.head_dim, dtype=w.dtype, device=xq.device)
+        fused = m.attend_on_page_stream and gather_attend_supported(
+            w.n_q_heads, w.n_kv_heads, w.head_dim, w.page_size, w.dtype)
+        blocks = max(1, min(GATHER_BLOCKS // w.n_kv_heads, idx.shape[1])) if fused else 0
+        if fused:   # the page stream that also attends over the pages it moves
+            timed("pages_gather", lambda: lru.gather_attend_(
+                idx.shape[1], xq[0, 0], 1.0 / math.sqrt(w.head_dim), m.cache_k.shape[1],
+                m._workspace, blocks))
+        else:
+            timed("pages_gather", lambda: lru.gather_(idx.shape[1]))
         for name, phase in (("decode_attention_split", PagedPrefix.FIRST),
                             ("decode_attention_first_merge", PagedPrefix.FIRST_MERGE),
                             ("decode_attention_tail+merge", PagedPrefix.SECOND)):
             timed(name, lambda phase=phase: decode_attention(
                 *args, workspace=m._workspace, out=out,
-                paged=PagedPrefix(w.page_size, scratch, lru.current_step, phase)))
+                paged=PagedPrefix(w.page_size, scratch, lru.current_step, phase, blocks)))
         torch.cuda.synchronize()
         for name, e0, e1, repeat in pending:
             acc[name] += e0.elapsed_time(e1) / repeat

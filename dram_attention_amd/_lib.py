@@ -69,6 +69,12 @@ SIGNATURES = {
          c_void_p, c_int64, c_float, c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p,
          c_void_p],
     ),
+    "da_pages_gather_attend": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p,
+         c_void_p, c_int, c_int, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_float, c_int64,
+         c_int64, c_void_p, c_size_t, c_void_p],
+    ),
 }
 
 
@@ -84,6 +90,7 @@ class PagedOverlap(ctypes.Structure):
         ("miss_slot", c_void_p),
         ("miss_count", c_void_p),
         ("miss_capacity", ctypes.c_int32),
+        ("gather_blocks", ctypes.c_int32),
     ]
 
 _lib = None

@@ -154,6 +154,8 @@ struct AttnArgs {
   int n_pchunks, n_lchunks, n_tchunks;
   int chunk_base;  // chunk id of blockIdx.x == 0 in this launch
   int pre_chunk;   // chunk id that holds the merged result of the prefix and local chunks
+  int gather_chunk0;   // first chunk id of the partials a gather-with-attention pass wrote
+  int gather_blocks;   // its blocks per kv head (0: the tail kernel covers the re-assigned slots)
   int n_q_heads;
   float *part_ml;   // (chunks, Hq, 2): running max (log2 domain), sum
   float *part_acc;  // (chunks, Hq, D)
@@ -429,7 +431,13 @@ decode_attention_merge_kernel(const AttnArgs a, int mode, int head_dim, char *__
   const int n_p = a.n_pchunks;                              // live prefix chunks (all of them)
   const int n_l = (int)((l_len + a.chunk - 1) / a.chunk);   // live local chunks
   int n_t = 0;                                              // live tail chunks
-  if (a.n_tchunks > 0 && mode != kMergePre) {
+  int tail_chunk0 = a.n_pchunks + a.n_lchunks;
+  if (a.gather_blocks > 0 && mode != kMergePre) {
+    // block b of the gather pass wrote a partial iff it had an entry to copy
+    const int misses = a.miss_count[hq / a.rep];
+    n_t = misses < a.gather_blocks ? misses : a.gather_blocks;
+    tail_chunk0 = a.gather_chunk0;
+  } else if (a.n_tchunks > 0 && mode != kMergePre) {
     const int64_t tail = (int64_t)a.miss_count[hq / a.rep] * a.page_size;
     n_t = (int)((tail + a.tail_chunk - 1) / a.tail_chunk);
   }
@@ -438,7 +446,7 @@ decode_attention_merge_kernel(const AttnArgs a, int mode, int head_dim, char *__
   // i-th live chunk -> chunk id
   auto chunk_of = [&](int i) {
     if (i < n_first) return mode == kMergeFinal ? a.pre_chunk : i;
-    return a.n_pchunks + a.n_lchunks + (i - n_first);
+    return tail_chunk0 + (i - n_first);
   };
 
   // Stage the (max, sum) pairs of the live chunks in LDS with one load per
@@ -535,11 +543,15 @@ static int lanes_of(int head_dim, int dtype) {
   return (lanes >= 4 && lanes <= 64 && is_pow2(lanes)) ? lanes : 0;
 }
 
+constexpr int kGatherMaxBlocks = 64;  // per kv head
+
 struct ChunkPlan {
   int chunk, tail_chunk, n_p, n_l, n_t;
-  // one more slot than there are chunks: the merged state of the first pass
-  int64_t total() const { return (int64_t)n_p + n_l + n_t + 1; }
+  // slots beyond the chunks: the merged state of the first pass, then (with a
+  // tail) one per block and kv head of a gather-with-attention pass
+  int64_t total() const { return (int64_t)n_p + n_l + n_t + 1 + (n_t > 0 ? kGatherMaxBlocks : 0); }
   int pre_chunk() const { return n_p + n_l + n_t; }
+  int gather_chunk0() const { return n_p + n_l + n_t + 1; }
 };
 // The chunk geometry of a launch; a function of the shapes only, so that the
 // workspace query and every phase of a step agree on it.
@@ -619,7 +631,9 @@ static int launch_attention(const AttnArgs &a, int phase, int n_kv_heads, int la
   if (phase & DA_PHASE_SECOND) {
     // everything in one call and no carried partial: one merge over all chunks
     const bool all = (phase & DA_PHASE_FIRST) && !(phase & DA_PHASE_FIRST_MERGE);
-    if (a.n_tchunks > 0) {
+    if (a.gather_blocks > 0) {
+      // the re-assigned slots were attended while they were copied
+    } else if (a.n_tchunks > 0) {
       DA_ATTN_LAUNCH(true, a.n_pchunks + a.n_lchunks, a.n_tchunks)
       int rc = launch_status("da_decode_attention(tail)");
       if (rc) return rc;
@@ -634,7 +648,293 @@ static int launch_attention(const AttnArgs &a, int phase, int n_kv_heads, int la
   return DA_OK;
 }
 
+
+// ---------------------------------------------------------------------------
+// Page stream with attention riding on it.  A block copies the pages of one kv
+// head's miss list (entries blockIdx.x, += gridDim.x) from the host page store
+// into their slots, 16 bytes per lane, and the registers the page passes
+// through also feed the attention of this step's query over that page: the
+// re-assigned slots then need no second pass after the stream has finished.
+// A page holds page_size tokens, each token its K row followed by its V row,
+// so 2*kLanes adjacent lanes hold one token: the lower kLanes its key (they
+// produce the score), the upper kLanes its value (they keep the softmax state
+// and the weighted sum).  The next page's loads are issued before the current
+// page is stored and attended, so the host link never waits for arithmetic.
+// Every block with an entry to copy leaves one partial (all query rows of the
+// kv head) at chunk id gather_chunk0 + blockIdx.x.
+struct GatherAttendArgs {
+  const char *dram;
+  int64_t dram_head_stride, dram_page_stride;
+  char *hbm;
+  int64_t hbm_head_stride, hbm_slot_stride;
+  int page_vecs;  // 16-byte lanes per page
+  const int32_t *miss_page, *miss_slot, *miss_count;
+  int K;
+  const char *q;
+  int64_t q_head_stride;
+  int rep, n_q_heads;
+  float scale_log2;
+  float *part_ml, *part_acc;
+  int chunk0;
+};
+
+constexpr int kGatherThreads = 256;
+constexpr int kGatherMaxLoads = 4;  // 16-byte loads per lane and page: pages up to 16 KiB
+constexpr int kGatherIdBatch = 1024;  // miss-list entries of a block staged in LDS at a time
+
+template <typename T, int kLanes, int kRows>
+__global__ void __launch_bounds__(kGatherThreads)
+pages_gather_attend_kernel(const GatherAttendArgs g) {
+  constexpr int V = T::kVec;
+  constexpr int D = kLanes * V;
+  constexpr int kTokLanes = 2 * kLanes;
+  constexpr int kWaves = kGatherThreads / 64;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int within = tid % kTokLanes;
+  const bool is_v = within >= kLanes;
+  const int c = within % kLanes;
+  const int h = blockIdx.y;
+  const int n_miss = g.miss_count[h];
+  if ((int)blockIdx.x >= n_miss) return;  // the merge does not count this block either
+
+  u32x4 qv[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const int rr = r < g.rep ? r : g.rep - 1;
+    qv[r] = load16(g.q + ((int64_t)(h * g.rep + rr) * g.q_head_stride) * T::kBytes + c * 16);
+  }
+  float m[kRows], l[kRows], acc[kRows][V];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    m[r] = kMinusHuge;
+    l[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[r][i] = 0.f;
+  }
+
+  const int32_t *mpage = g.miss_page + (int64_t)h * g.K;
+  const int32_t *mslot = g.miss_slot + (int64_t)h * g.K;
+  // This block's entries (slot, page), staged in LDS a batch at a time: a page's
+  // loads then depend on no other global load, and the next page is always in
+  // flight while the current one is stored and attended.
+  __shared__ int32_t sm_slot[kGatherIdBatch], sm_page[kGatherIdBatch];
+  const int n_mine = (n_miss - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  // Issues the loads of this block's n-th staged entry; dst == nullptr marks a
+  // superseded one.  Always kGatherMaxLoads loads per lane, lanes with nothing to
+  // fetch reading the query instead: with a fixed count the wait for one page's
+  // data can leave the next page's loads outstanding.
+  auto fetch = [&](int n, int n_batch, u32x4 *buf, char *&dst) {
+    const bool real = n < n_batch;  // past the batch: the same loads, all of them idle
+    const int32_t v = real ? sm_slot[n] : -1;
+    const int32_t p = real ? sm_page[n] : 0;
+    const char *src = g.dram + h * g.dram_head_stride + p * g.dram_page_stride;
+    dst = v < 0 ? nullptr : g.hbm + h * g.hbm_head_stride + v * g.hbm_slot_stride;
+#pragma unroll
+    for (int u = 0; u < kGatherMaxLoads; ++u) {
+      const int j = u * kGatherThreads + tid;
+      buf[u] = load16(v >= 0 && j < g.page_vecs ? src + (int64_t)j * 16 : g.q);
+    }
+  };
+  auto settle = [&](const u32x4 *buf, char *dst) {
+    if (dst == nullptr) return;
+#pragma unroll
+    for (int u = 0; u < kGatherMaxLoads; ++u) {
+      const int j = u * kGatherThreads + tid;
+      if (j < g.page_vecs) store16(dst + (int64_t)j * 16, buf[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kGatherMaxLoads; ++u) {
+      if (u * kGatherThreads >= g.page_vecs) continue;  // uniform
+      const bool tok = u * kGatherThreads + tid < g.page_vecs;
+      const u32x4 data = tok ? buf[u] : u32x4{0, 0, 0, 0};
+      float vf[V];
+      unpack<T>(data, vf);
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        const float sk = group_sum<kLanes>(dot16<T>(qv[r], data)) * g.scale_log2;
+        const float so = __shfl_xor(sk, kLanes, 64);  // a value lane takes its key lane's
+        float sc = is_v ? so : sk;
+        if (!tok) sc = -INFINITY;
+        const float mn = fmaxf(m[r], sc);
+        const float alpha = fast_exp2(m[r] - mn);
+        const float pw = fast_exp2(sc - mn);
+        m[r] = mn;
+        l[r] = l[r] * alpha + pw;
+#pragma unroll
+        for (int x = 0; x < V; ++x) acc[r][x] = acc[r][x] * alpha + pw * vf[x];
+      }
+    }
+  };
+
+  for (int batch0 = 0; batch0 < n_mine; batch0 += kGatherIdBatch) {
+    const int n_batch = n_mine - batch0 < kGatherIdBatch ? n_mine - batch0 : kGatherIdBatch;
+    __syncthreads();  // the previous batch is no longer read
+    for (int n = tid; n < n_batch; n += kGatherThreads) {
+      const int64_t i = (int64_t)blockIdx.x + (int64_t)(batch0 + n) * gridDim.x;
+      sm_slot[n] = mslot[i];
+      sm_page[n] = mpage[i];
+    }
+    __syncthreads();
+    // two page buffers in turn: one is stored and attended while the other fills
+    u32x4 a_buf[kGatherMaxLoads], b_buf[kGatherMaxLoads];
+    char *a_dst = nullptr, *b_dst = nullptr;
+    fetch(0, n_batch, a_buf, a_dst);
+    for (int n = 0; n < n_batch; n += 2) {
+      fetch(n + 1, n_batch, b_buf, b_dst);
+      settle(a_buf, a_dst);
+      fetch(n + 2, n_batch, a_buf, a_dst);
+      settle(b_buf, b_dst);
+    }
+  }
+
+  // Merge the tokens of a wave (lanes of equal position within a token pair up).
+#pragma unroll
+  for (int off = kTokLanes; off < 64; off <<= 1) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const float mo = __shfl_xor(m[r], off, 64);
+      const float lo = __shfl_xor(l[r], off, 64);
+      const float mn = fmaxf(m[r], mo);
+      const float wa = fast_exp2(m[r] - mn), wb = fast_exp2(mo - mn);
+      l[r] = l[r] * wa + lo * wb;
+#pragma unroll
+      for (int x = 0; x < V; ++x) {
+        const float ao = __shfl_xor(acc[r][x], off, 64);
+        acc[r][x] = acc[r][x] * wa + ao * wb;
+      }
+      m[r] = mn;
+    }
+  }
+  // Merge the waves through LDS; the value lanes of a wave's first token hold its state.
+  __shared__ float sm_m[kWaves][kRows];
+  __shared__ float sm_l[kWaves][kRows];
+  __shared__ float sm_acc[kWaves][kRows][D];
+  if (is_v && lane < kTokLanes) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      if (c == 0) {
+        sm_m[wave][r] = m[r];
+        sm_l[wave][r] = l[r];
+      }
+#pragma unroll
+      for (int x = 0; x < V; ++x) sm_acc[wave][r][c * V + x] = acc[r][x];
+    }
+  }
+  __syncthreads();
+  const int chunk_id = g.chunk0 + blockIdx.x;
+  for (int item = tid; item < kRows * D; item += kGatherThreads) {
+    const int r = item / D, d = item % D;
+    if (r >= g.rep) continue;
+    float mn = sm_m[0][r];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mn = fmaxf(mn, sm_m[w][r]);
+    float lt = 0.f, at = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float wgt = fast_exp2(sm_m[w][r] - mn);
+      lt += sm_l[w][r] * wgt;
+      at += sm_acc[w][r][d] * wgt;
+    }
+    const int64_t slot = (int64_t)chunk_id * g.n_q_heads + (int64_t)h * g.rep + r;
+    g.part_acc[slot * D + d] = at;
+    if (d == 0) {
+      g.part_ml[slot * 2] = mn;
+      g.part_ml[slot * 2 + 1] = lt;
+    }
+  }
+}
+
+template <typename T, int kLanes>
+static void launch_gather_attend(const GatherAttendArgs &g, dim3 grid, hipStream_t s) {
+  if (g.rep <= 4)
+    hipLaunchKernelGGL((pages_gather_attend_kernel<T, kLanes, 4>), grid, dim3(kGatherThreads), 0, s,
+                       g);
+  else
+    hipLaunchKernelGGL((pages_gather_attend_kernel<T, kLanes, 8>), grid, dim3(kGatherThreads), 0, s,
+                       g);
+}
+
+template <typename T>
+static int dispatch_gather_attend(const GatherAttendArgs &g, int lanes, dim3 grid, hipStream_t s) {
+  switch (lanes) {
+    case 4: launch_gather_attend<T, 4>(g, grid, s); break;
+    case 8: launch_gather_attend<T, 8>(g, grid, s); break;
+    case 16: launch_gather_attend<T, 16>(g, grid, s); break;
+    case 32: launch_gather_attend<T, 32>(g, grid, s); break;
+    default: return fail(DA_ENOTSUP, "da_pages_gather_attend: rows of %d bytes", lanes * 16);
+  }
+  return launch_status("da_pages_gather_attend");
+}
+
 }  // namespace da
+
+extern "C" int da_pages_gather_attend(
+    const void *dram, int64_t dram_head_stride_bytes, int64_t dram_page_stride_bytes, void *hbm,
+    int64_t hbm_head_stride_bytes, int64_t hbm_slot_stride_bytes, int page_size,
+    const int32_t *miss_page, const int32_t *miss_slot, const int32_t *miss_count, int n_kv_heads,
+    int k, int blocks_per_head, const void *q, int64_t q_head_stride, int n_q_heads, int head_dim,
+    int dtype, float scale, int64_t p_len, int64_t c_capacity, void *workspace,
+    size_t workspace_bytes, void *stream) {
+  using namespace da;
+  DA_REQUIRE(n_kv_heads > 0 && n_q_heads > 0 && n_q_heads % n_kv_heads == 0 && k > 0 &&
+                 page_size > 0 && p_len >= 0 && c_capacity >= 0,
+             "da_pages_gather_attend: bad geometry");
+  DA_REQUIRE(dtype == DA_F32 || dtype == DA_F16 || dtype == DA_BF16,
+             "da_pages_gather_attend: unknown dtype %d", dtype);
+  DA_REQUIRE(dram && hbm && miss_page && miss_slot && miss_count && q && workspace,
+             "da_pages_gather_attend: null pointer");
+  DA_REQUIRE(blocks_per_head >= 1 && blocks_per_head <= kGatherMaxBlocks,
+             "da_pages_gather_attend: blocks_per_head %d not in 1..%d", blocks_per_head,
+             kGatherMaxBlocks);
+  const int lanes = lanes_of(head_dim, dtype);
+  const int rep = n_q_heads / n_kv_heads;
+  const int64_t page_vecs = (int64_t)page_size * 2 * lanes;
+  if (!lanes || lanes > 32 || rep > 8 || page_vecs > kGatherThreads * kGatherMaxLoads ||
+      n_kv_heads > 65535)
+    return fail(DA_ENOTSUP,
+                "da_pages_gather_attend: needs rows of 64..512 bytes, at most 8 query heads per kv "
+                "head and pages up to %d bytes (use da_pages_gather and the tail pass instead)",
+                kGatherThreads * kGatherMaxLoads * 16);
+  const int vec = dtype == DA_F32 ? 4 : 8;
+  DA_REQUIRE(dram_head_stride_bytes % 16 == 0 && dram_page_stride_bytes % 16 == 0 &&
+                 hbm_head_stride_bytes % 16 == 0 && hbm_slot_stride_bytes % 16 == 0 &&
+                 (uintptr_t)dram % 16 == 0 && (uintptr_t)hbm % 16 == 0 && (uintptr_t)q % 16 == 0 &&
+                 q_head_stride % vec == 0 && (uintptr_t)workspace % 16 == 0,
+             "da_pages_gather_attend: operands must be 16-byte aligned");
+  const ChunkPlan p = plan_chunks(n_kv_heads, lanes, p_len, c_capacity, (int64_t)k * page_size);
+  const size_t need = attn_workspace_bytes(n_q_heads, head_dim, p.total());
+  DA_REQUIRE(workspace_bytes >= need, "da_pages_gather_attend: workspace %zu < %zu bytes",
+             workspace_bytes, need);
+  GatherAttendArgs g = {};
+  g.dram = (const char *)dram;
+  g.dram_head_stride = dram_head_stride_bytes;
+  g.dram_page_stride = dram_page_stride_bytes;
+  g.hbm = (char *)hbm;
+  g.hbm_head_stride = hbm_head_stride_bytes;
+  g.hbm_slot_stride = hbm_slot_stride_bytes;
+  g.page_vecs = (int)page_vecs;
+  g.miss_page = miss_page;
+  g.miss_slot = miss_slot;
+  g.miss_count = miss_count;
+  g.K = k;
+  g.q = (const char *)q;
+  g.q_head_stride = q_head_stride;
+  g.rep = rep;
+  g.n_q_heads = n_q_heads;
+  g.scale_log2 = scale * kLog2e;
+  g.part_acc = (float *)workspace;
+  g.part_ml = g.part_acc + (size_t)p.total() * n_q_heads * head_dim;
+  g.chunk0 = p.gather_chunk0();
+  const dim3 grid(blocks_per_head, n_kv_heads);
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case DA_F32: return dispatch_gather_attend<F32>(g, lanes, grid, s);
+    case DA_F16: return dispatch_gather_attend<F16>(g, lanes, grid, s);
+    default: return dispatch_gather_attend<BF16>(g, lanes, grid, s);
+  }
+}
 
 extern "C" size_t da_decode_attention_workspace_bytes(int n_q_heads, int n_kv_heads,
                                                       int head_dim, int dtype, int64_t p_len,
@@ -732,6 +1032,11 @@ extern "C" int da_decode_attention_paged(
     a.miss_capacity = overlap->miss_capacity;
     miss_tokens = (int64_t)overlap->miss_capacity * overlap->page_size;
     phase = overlap->phase;
+    DA_REQUIRE(overlap->gather_blocks >= 0 && overlap->gather_blocks <= kGatherMaxBlocks &&
+                   (overlap->gather_blocks == 0 || miss_tokens > 0),
+               "da_decode_attention: gather_blocks %d out of range (at most %d)",
+               overlap->gather_blocks, kGatherMaxBlocks);
+    a.gather_blocks = overlap->gather_blocks;
   }
   const ChunkPlan p = plan_chunks(n_kv_heads, lanes, p_len, c_capacity, miss_tokens);
   a.chunk = p.chunk;
@@ -740,6 +1045,7 @@ extern "C" int da_decode_attention_paged(
   a.n_lchunks = p.n_l;
   a.n_tchunks = p.n_t;
   a.pre_chunk = p.pre_chunk();
+  a.gather_chunk0 = p.gather_chunk0();
   const size_t need = attn_workspace_bytes(n_q_heads, head_dim, p.total());
   DA_REQUIRE(workspace_bytes >= need, "da_decode_attention: workspace %zu < %zu bytes",
              workspace_bytes, need);

@@ -17,6 +17,7 @@ import torch.nn.functional as F
 
 from . import _lib
 from .lru_cache import DummyCache, LRUCache
+from .lru_kernel import GATHER_BLOCKS, gather_attend_supported
 
 
 class PagedPrefix:
@@ -30,11 +31,15 @@ class PagedPrefix:
 
     FIRST, SECOND, FIRST_MERGE = 1, 2, 4
 
-    def __init__(self, page_size: int, scratch, current_step: torch.Tensor, phase: int):
+    def __init__(self, page_size: int, scratch, current_step: torch.Tensor, phase: int,
+                 gather_blocks: int = 0):
         self.page_size = page_size
         self.scratch = scratch
         self.current_step = current_step
         self.phase = phase
+        # blocks per kv head of a pages_gather_attend stream that already covered
+        # the re-assigned slots (0: the SECOND pass attends over them)
+        self.gather_blocks = gather_blocks
 
     def as_struct(self) -> "_lib.PagedOverlap":
         s = self.scratch
@@ -42,7 +47,7 @@ class PagedPrefix:
             page_size=self.page_size, phase=self.phase, slot_epoch=s.slot_epoch.data_ptr(),
             slot_epoch_head_stride=s.slot_epoch.stride(0), epoch=self.current_step.data_ptr(),
             miss_slot=s.miss_slot.data_ptr(), miss_count=s.miss_count.data_ptr(),
-            miss_capacity=s.miss_slot.shape[1])
+            miss_capacity=s.miss_slot.shape[1], gather_blocks=self.gather_blocks)
 
 
 def attention_workspace(Hq: int, Hkv: int, D: int, dtype: torch.dtype, p_len: int, capacity: int,
@@ -201,6 +206,9 @@ class DRAMAttention(torch.nn.Module):
         self._side_stream = None
         # stream missed pages on a side stream underneath the attention pass
         self.overlap_page_stream = True
+        # attend over the streamed pages inside the page stream itself (when the
+        # shape allows) instead of a pass over them after the stream
+        self.attend_on_page_stream = True
 
     def init_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor):
         """Split the prompt's (1,S,Hkv,D) keys/values into the paged prefix and the
@@ -276,14 +284,31 @@ class DRAMAttention(torch.nn.Module):
                 scratch.miss_slot.shape[1] * self.page_size, xq.device)
         args = (xq[0, 0], prefix_k, prefix_v, self.cache_k[0], self.cache_v[0], cache_len,
                 xk[0, 0], xv[0, 0])
-        if not self.overlap_page_stream:
-            lru.gather_(idx.shape[1])
+        k = idx.shape[1]
+        # Attention over the pages paged in this step rides on the page stream when
+        # the shape allows; otherwise a tail pass covers them after the stream.
+        fused = self.attend_on_page_stream and gather_attend_supported(
+            Hq, self.n_kv_heads, D, self.page_size, xq.dtype)
+        blocks = max(1, min(GATHER_BLOCKS // self.n_kv_heads, k)) if fused else 0
+
+        def stream_pages():
+            if fused:
+                lru.gather_attend_(k, xq[0, 0], 1.0 / math.sqrt(D), self.cache_k.shape[1],
+                                   self._workspace, blocks)
+            else:
+                lru.gather_(k)
+
+        def attend(phase):
             decode_attention(*args, workspace=self._workspace, out=out[0, 0],
                              cache_len_offset=offset,
-                             # the same kernels as the overlapped order, so the same bits
-                             paged=PagedPrefix(self.page_size, scratch, lru.current_step,
-                                               PagedPrefix.FIRST | PagedPrefix.FIRST_MERGE |
-                                               PagedPrefix.SECOND))
+                             paged=PagedPrefix(self.page_size, scratch, lru.current_step, phase,
+                                               blocks))
+
+        P = PagedPrefix
+        if not self.overlap_page_stream:
+            stream_pages()
+            # the same kernels as the overlapped order, so the same bits
+            attend(P.FIRST | P.FIRST_MERGE | P.SECOND)
             return out
         main = torch.cuda.current_stream(xq.device)
         if self._side_stream is None:
@@ -291,12 +316,8 @@ class DRAMAttention(torch.nn.Module):
         side = self._side_stream
         side.wait_stream(main)                      # the miss list is ready
         with torch.cuda.stream(side):
-            lru.gather_(idx.shape[1])
-        decode_attention(*args, workspace=self._workspace, out=out[0, 0], cache_len_offset=offset,
-                         paged=PagedPrefix(self.page_size, scratch, lru.current_step,
-                                           PagedPrefix.FIRST | PagedPrefix.FIRST_MERGE))
+            stream_pages()
+        attend(P.FIRST | P.FIRST_MERGE)
         main.wait_stream(side)                      # the pages have landed
-        decode_attention(*args, workspace=self._workspace, out=out[0, 0], cache_len_offset=offset,
-                         paged=PagedPrefix(self.page_size, scratch, lru.current_step,
-                                           PagedPrefix.SECOND))
+        attend(P.SECOND)
         return out

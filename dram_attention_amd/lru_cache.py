@@ -12,7 +12,8 @@ from typing import NamedTuple, Optional
 import torch
 
 from . import _lib
-from .lru_kernel import LruScratch, lru_update, lru_update_and_gather, pages_gather
+from .lru_kernel import (LruScratch, lru_update, lru_update_and_gather, pages_gather,
+                         pages_gather_attend)
 from .topk_selector import IPUpperboundTopKSelector
 
 
@@ -180,6 +181,15 @@ class LRUCache(torch.nn.Module):
             self._dram_device_ptr = _lib.device_visible_ptr(self.dram_kv_cache)
         pages_gather(self.dram_kv_cache, self.hbm_kv_cache, self._scratch, k,
                      self._dram_device_ptr)
+
+    def gather_attend_(self, k: int, xq: torch.Tensor, scale: float, c_capacity: int,
+                       workspace: torch.Tensor, blocks_per_head: int) -> None:
+        """gather_ with the step's attention over the streamed pages computed on the way."""
+        if self._dram_device_ptr is None:
+            self._dram_device_ptr = _lib.device_visible_ptr(self.dram_kv_cache)
+        pages_gather_attend(self.dram_kv_cache, self.hbm_kv_cache, self._scratch, k,
+                            self.page_size, xq, scale, self.num_hbm_pages * self.page_size,
+                            c_capacity, workspace, blocks_per_head, self._dram_device_ptr)
 
     def views(self) -> CacheOutput:
         return self._views()

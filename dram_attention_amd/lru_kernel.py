@@ -119,6 +119,46 @@ def pages_gather(dram_kv_cache: torch.Tensor, hbm_kv_cache: torch.Tensor, scratc
     )
 
 
+GATHER_BLOCKS = 32  # workgroups of a page stream in all: few and fat saturate the host link
+
+
+def gather_attend_supported(n_q_heads: int, n_kv_heads: int, head_dim: int, page_size: int,
+                            dtype: torch.dtype) -> bool:
+    """Whether pages_gather_attend takes this shape (else: pages_gather + tail pass)."""
+    row = head_dim * torch.empty(0, dtype=dtype).element_size()
+    return (row in (64, 128, 256, 512) and n_q_heads // n_kv_heads <= 8
+            and page_size * 2 * row <= 16384)
+
+
+def pages_gather_attend(dram_kv_cache: torch.Tensor, hbm_kv_cache: torch.Tensor,
+                        scratch: LruScratch, k: int, page_size: int, xq: torch.Tensor,
+                        scale: float, p_len: int, c_capacity: int, workspace: torch.Tensor,
+                        blocks_per_head: int, dram_device_ptr: Optional[int] = None) -> None:
+    """pages_gather, with the attention of query ``xq`` (Hq, D) over every copied
+    page computed on the way; the partial results land in ``workspace`` (the one
+    the step's decode_attention calls use) for the final merge."""
+    num_heads = dram_kv_cache.shape[0]
+    Hq, D = xq.shape
+    if dram_device_ptr is None:
+        dram_device_ptr = _lib.device_visible_ptr(dram_kv_cache)
+    esz = dram_kv_cache.element_size()
+    if dram_kv_cache.shape[2] != page_size * 2 * D or xq.dtype != hbm_kv_cache.dtype:
+        raise ValueError("pages must hold page_size tokens of (K row, V row) in the query's dtype")
+    lib = _lib.load()
+    _lib.check(
+        lib.da_pages_gather_attend(
+            dram_device_ptr, dram_kv_cache.stride(0) * esz, dram_kv_cache.stride(1) * esz,
+            hbm_kv_cache.data_ptr(), hbm_kv_cache.stride(0) * esz, hbm_kv_cache.stride(1) * esz,
+            page_size, scratch.miss_page.data_ptr(), scratch.miss_slot.data_ptr(),
+            scratch.miss_count.data_ptr(), num_heads, k, blocks_per_head,
+            xq.data_ptr(), xq.stride(0), Hq, D, _lib.dtype_code(xq.dtype), scale, p_len,
+            c_capacity, workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+            _lib.stream_ptr(hbm_kv_cache.device),
+        ),
+        "da_pages_gather_attend",
+    )
+
+
 def lru_update_and_gather(
     dram_kv_cache: torch.Tensor,
     page_access_time: torch.Tensor,

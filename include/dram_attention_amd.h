@@ -218,6 +218,9 @@ int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
  *                          after the page stream has completed.  Without
  *                          DA_PHASE_FIRST in the same call it merges the tail with
  *                          the partial DA_PHASE_FIRST_MERGE left in the workspace.
+ * When the page stream of the step was da_pages_gather_attend, which attends
+ * over the re-assigned slots itself, set `gather_blocks` to its
+ * blocks_per_head: DA_PHASE_SECOND is then only the final merge.
  * The usual step: FIRST | FIRST_MERGE next to the stream, SECOND after the join.
  * FIRST | SECOND in one call (the page stream already complete) needs no
  * FIRST_MERGE.
@@ -237,6 +240,7 @@ typedef struct da_paged_overlap {
   const int32_t *miss_slot;       /* (Hkv, miss_capacity) */
   const int32_t *miss_count;      /* (Hkv) */
   int32_t miss_capacity;
+  int32_t gather_blocks;          /* blocks_per_head of da_pages_gather_attend, else 0 */
 } da_paged_overlap;
 
 int da_decode_attention_paged(const void *q, int64_t q_head_stride, int n_q_heads,
@@ -249,6 +253,36 @@ int da_decode_attention_paged(const void *q, int64_t q_head_stride, int n_q_head
                               int64_t out_head_stride, float *lse_out, void *workspace,
                               size_t workspace_bytes, const da_paged_overlap *overlap,
                               void *stream);
+
+/*
+ * Subsystem 4b + 5 — the page stream with this step's attention riding on it
+ * (no counterpart in the reference, which copies pages first and attends
+ * afterwards, dram_attention/lru_triton_kernel.py:80-98 then
+ * dram_attention/dram_attention.py:191-238).  Copies exactly what
+ * da_pages_gather copies; the registers a page passes through also feed the
+ * attention of query `q` over that page, so that the step needs no second pass
+ * over the re-assigned slots once the stream has finished.
+ *   page layout : page_size tokens, each token its K row (head_dim) followed by
+ *                 its V row; dram / hbm strides in bytes as for da_pages_gather
+ *   q           : (Hq, head_dim), element stride q_head_stride
+ *   workspace   : the workspace of this step's da_decode_attention_paged calls
+ *                 (same p_len, c_capacity, and miss_capacity = k); every block
+ *                 with an entry to copy leaves one partial result in it
+ *   blocks_per_head : workgroups per kv head, 1..64 (few fat ones: 32 in all
+ *                 saturate the host link); pass the same value as
+ *                 da_paged_overlap.gather_blocks to DA_PHASE_SECOND
+ * DA_ENOTSUP when rows are not 64..512 bytes, Hq / Hkv > 8 or a page exceeds
+ * 16 KiB: use da_pages_gather and the tail pass of DA_PHASE_SECOND then.
+ */
+int da_pages_gather_attend(const void *dram, int64_t dram_head_stride_bytes,
+                           int64_t dram_page_stride_bytes, void *hbm,
+                           int64_t hbm_head_stride_bytes, int64_t hbm_slot_stride_bytes,
+                           int page_size, const int32_t *miss_page, const int32_t *miss_slot,
+                           const int32_t *miss_count, int n_kv_heads, int k,
+                           int blocks_per_head, const void *q, int64_t q_head_stride,
+                           int n_q_heads, int head_dim, int dtype, float scale, int64_t p_len,
+                           int64_t c_capacity, void *workspace, size_t workspace_bytes,
+                           void *stream);
 
 #ifdef __cplusplus
 }

@@ -243,6 +243,50 @@ def test_page_stream_overlap_changes_nothing():
         assert close(plain, b[0, 0], 1e-2, 1e-2)
 
 
+@pytest.mark.parametrize("base,kw", [
+    ("128k", dict(dram_tokens=16384, local_cache=1024, lru_tokens=4096, top_k_tokens=1024, steps=5)),
+    ("1m", dict(dram_tokens=8192, local_cache=512, lru_tokens=2048, top_k_tokens=256, steps=4,
+                planted_pages=8)),
+    ("cpu", dict(steps=4)),
+    ("128k", dict(dram_tokens=8192, local_cache=512, lru_tokens=2048, top_k_tokens=512, steps=4,
+                  page_size=32, dtype=torch.float16)),
+    ("128k", dict(dram_tokens=4096, local_cache=256, lru_tokens=1024, top_k_tokens=128, steps=4,
+                  page_size=8, head_dim=64, n_q_heads=4, n_kv_heads=2)),
+])
+def test_attention_on_the_page_stream_equals_tail_pass(base, kw):
+    """Attending over the streamed pages inside the page stream, or in a pass
+    over them afterwards: the same slots, maps and cache rows bit for bit, and
+    the same output up to the order of the softmax merge."""
+    from dram_attention_amd import DRAMAttention
+    from dram_attention_amd.lru_kernel import gather_attend_supported
+
+    w = WORKLOADS[base].scaled(**kw)
+    assert gather_attend_supported(w.n_q_heads, w.n_kv_heads, w.head_dim, w.page_size, w.dtype)
+    prompt = make_prompt(w, 8)
+    mods = []
+    for fused in (True, False):
+        m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                          w.n_kv_heads, w.head_dim, device=DEV, dtype=w.dtype)
+        m.attend_on_page_stream = fused
+        m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+        mods.append(m)
+    inputs = DecodeInputs(w, prompt.q0, 8)
+    atol, rtol = (1e-5, 1e-4) if w.dtype == torch.float32 else (1e-2, 1e-2)
+    misses = 0
+    for t in range(w.steps):
+        xq, xk, xv = (x.to(DEV) for x in inputs.next())
+        a = mods[0](xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
+        b = mods[1](xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
+        torch.cuda.synchronize()
+        misses += mods[0].lru_cache.last_miss_counts().sum().item()
+        assert close(a.float(), b.float(), atol, rtol), f"step {t}"
+        la, lb = mods[0].lru_cache, mods[1].lru_cache
+        assert same(la.hbm_kv_cache, lb.hbm_kv_cache), f"slots, step {t}"
+        assert same(la.dram_page_to_hbm_page_mapping, lb.dram_page_to_hbm_page_mapping)
+        assert same(mods[0].cache_k, mods[1].cache_k)
+    assert misses > 0
+
+
 def test_graph_replay_equals_eager_steps():
     """The whole step (selection, LRU, page stream on its side stream, two-phase
     attention, append) captured once and replayed: every replay, with eager work
