@@ -117,7 +117,7 @@ def time_kernels(layer, steps):
 
     m, lru, w = layer.m, layer.m.lru_cache, layer.w
     names = ("page_score", "topk_pages", "lru_update", "pages_gather", "decode_attention_split",
-             "decode_attention_first_merge", "decode_attention_tail+merge")
+             "split+merge", "decode_attention_first_merge", "decode_attention_tail+merge")
     acc = {n: 0.0 for n in names}
     misses, local_rows = 0, []
     if not isinstance(lru, LRUCache):
@@ -176,9 +176,16 @@ def time_kernels(layer, steps):
                 m._workspace, blocks))
         else:
             timed("pages_gather", lambda: lru.gather_(idx.shape[1]))
-        for name, phase in (("decode_attention_split", PagedPrefix.FIRST),
-                            ("decode_attention_first_merge", PagedPrefix.FIRST_MERGE),
-                            ("decode_attention_tail+merge", PagedPrefix.SECOND)):
+        P = PagedPrefix
+        # fused stream: the step merges once, after the combined launch; its cost is
+        # (first pass + merge) - (first pass).  Otherwise: first-pass merge, then
+        # tail pass + final merge after the stream.
+        phases = ((("decode_attention_split", P.FIRST), ("split+merge", P.FIRST | P.SECOND))
+                  if fused else
+                  (("decode_attention_split", P.FIRST),
+                   ("decode_attention_first_merge", P.FIRST_MERGE),
+                   ("decode_attention_tail+merge", P.SECOND)))
+        for name, phase in phases:
             timed(name, lambda phase=phase: decode_attention(
                 *args, workspace=m._workspace, out=out,
                 paged=PagedPrefix(w.page_size, scratch, lru.current_step, phase, blocks)))
@@ -188,8 +195,10 @@ def time_kernels(layer, steps):
         misses += int(lru.last_miss_counts().sum().item())
         local_rows.append(c_len)
         layer.ctr += 1
-    return ({n: v / steps * 1e3 for n, v in acc.items()},  # microseconds
-            misses / steps, sum(local_rows) / len(local_rows))
+    us = {n: v / steps * 1e3 for n, v in acc.items() if v > 0.0}  # microseconds
+    if "split+merge" in us:
+        us["decode_attention_merge"] = us.pop("split+merge") - us["decode_attention_split"]
+    return us, misses / steps, sum(local_rows) / len(local_rows)
 
 
 def host_link_gbps(dev, mb=64, reps=5):
@@ -319,7 +328,7 @@ def main():
                         f"{w.dram_tokens}-token prefix in pinned host DRAM ({w.n_dram_pages} pages/head), "
                         f"local {w.local_cache}, LRU {w.lru_tokens} tokens, top-k {w.top_k_tokens} tokens",
             "launch": "eager" if args.eager else "hip-graph replay",
-            "page_stream": "serialised" if args.no_overlap else "side stream under attention",
+            "page_stream": "serialised" if args.no_overlap else "in the launch of the first attention pass",
             "seed": args.seed,
         },
         "roofline": {

@@ -91,6 +91,13 @@ class PagedOverlap(ctypes.Structure):
         ("miss_count", c_void_p),
         ("miss_capacity", ctypes.c_int32),
         ("gather_blocks", ctypes.c_int32),
+        ("dram", c_void_p),
+        ("dram_head_stride_bytes", c_int64),
+        ("dram_page_stride_bytes", c_int64),
+        ("hbm", c_void_p),
+        ("hbm_head_stride_bytes", c_int64),
+        ("hbm_slot_stride_bytes", c_int64),
+        ("miss_page", c_void_p),
     ]
 
 _lib = None

@@ -186,8 +186,7 @@ __device__ __forceinline__ LocalLen local_len(const AttnArgs &a) {
 // kTail = false: chunks of the prefix and local segments; kTail = true: chunks
 // of the tail segment (the slots listed in the miss list).
 template <typename T, int kLanes, int kRows, bool kTail>
-__global__ void __launch_bounds__(kAttnThreads)
-decode_attention_split_kernel(const AttnArgs a) {
+__device__ __forceinline__ void attention_split_block(const AttnArgs &a, const int block_x) {
   constexpr int V = T::kVec;
   constexpr int kGroups = 64 / kLanes;  // tokens per wave step
   constexpr int kStepTokens = kAttnWaves * kGroups;
@@ -200,7 +199,7 @@ decode_attention_split_kernel(const AttnArgs a) {
   const int h = blockIdx.y;
   const int row_group = blockIdx.z;
   const int row0 = row_group * kRows;  // first query row of the GQA group handled here
-  const int chunk_id = a.chunk_base + blockIdx.x;
+  const int chunk_id = a.chunk_base + block_x;
 
   // Which segment, which token range.
   const int kind = kTail ? 2 : (chunk_id < a.n_pchunks ? 0 : 1);
@@ -406,6 +405,231 @@ decode_attention_split_kernel(const AttnArgs a) {
   }
 }
 
+template <typename T, int kLanes, int kRows, bool kTail>
+__global__ void __launch_bounds__(kAttnThreads)
+decode_attention_split_kernel(const AttnArgs a) {
+  attention_split_block<T, kLanes, kRows, kTail>(a, blockIdx.x);
+}
+
+// ---------------------------------------------------------------------------
+// Page stream with attention riding on it.  A block copies the pages of one kv
+// head's miss list (entries block_x, += n_blocks) from the host page store
+// into their slots, 16 bytes per lane, and the registers the page passes
+// through also feed the attention of this step's query over that page: the
+// re-assigned slots then need no second pass after the stream has finished.
+// A page holds page_size tokens, each token its K row followed by its V row,
+// so 2*kLanes adjacent lanes hold one token: the lower kLanes its key (they
+// produce the score), the upper kLanes its value (they keep the softmax state
+// and the weighted sum).  The next page's loads are issued before the current
+// page is stored and attended, so the host link never waits for arithmetic.
+// Every block with an entry to copy leaves one partial (all query rows of the
+// kv head) at chunk id gather_chunk0 + block_x.
+struct GatherAttendArgs {
+  const char *dram;
+  int64_t dram_head_stride, dram_page_stride;
+  char *hbm;
+  int64_t hbm_head_stride, hbm_slot_stride;
+  int page_vecs;  // 16-byte lanes per page
+  const int32_t *miss_page, *miss_slot, *miss_count;
+  int K;
+  const char *q;
+  int64_t q_head_stride;
+  int rep, n_q_heads;
+  float scale_log2;
+  float *part_ml, *part_acc;
+  int chunk0;
+};
+
+constexpr int kGatherThreads = 256;
+constexpr int kGatherMaxLoads = 4;  // 16-byte loads per lane and page: pages up to 16 KiB
+constexpr int kGatherIdBatch = 1024;  // miss-list entries of a block staged in LDS at a time
+
+template <typename T, int kLanes, int kRows>
+__device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, const int block_x,
+                                                    const int n_blocks) {
+  constexpr int V = T::kVec;
+  constexpr int D = kLanes * V;
+  constexpr int kTokLanes = 2 * kLanes;
+  constexpr int kWaves = kGatherThreads / 64;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int within = tid % kTokLanes;
+  const bool is_v = within >= kLanes;
+  const int c = within % kLanes;
+  const int h = blockIdx.y;
+  const int n_miss = g.miss_count[h];
+  if (block_x >= n_miss) return;  // the merge does not count this block either
+
+  u32x4 qv[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const int rr = r < g.rep ? r : g.rep - 1;
+    qv[r] = load16(g.q + ((int64_t)(h * g.rep + rr) * g.q_head_stride) * T::kBytes + c * 16);
+  }
+  float m[kRows], l[kRows], acc[kRows][V];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    m[r] = kMinusHuge;
+    l[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[r][i] = 0.f;
+  }
+
+  const int32_t *mpage = g.miss_page + (int64_t)h * g.K;
+  const int32_t *mslot = g.miss_slot + (int64_t)h * g.K;
+  // This block's entries (slot, page), staged in LDS a batch at a time: a page's
+  // loads then depend on no other global load, and the next page is always in
+  // flight while the current one is stored and attended.
+  __shared__ int32_t sm_slot[kGatherIdBatch], sm_page[kGatherIdBatch];
+  const int n_mine = (n_miss - block_x + n_blocks - 1) / n_blocks;
+  // Issues the loads of this block's n-th staged entry; dst == nullptr marks a
+  // superseded one.  Always kGatherMaxLoads loads per lane, lanes with nothing to
+  // fetch reading the query instead: with a fixed count the wait for one page's
+  // data can leave the next page's loads outstanding.
+  auto fetch = [&](int n, int n_batch, u32x4 *buf, char *&dst) {
+    const bool real = n < n_batch;  // past the batch: the same loads, all of them idle
+    const int32_t v = real ? sm_slot[n] : -1;
+    const int32_t p = real ? sm_page[n] : 0;
+    const char *src = g.dram + h * g.dram_head_stride + p * g.dram_page_stride;
+    dst = v < 0 ? nullptr : g.hbm + h * g.hbm_head_stride + v * g.hbm_slot_stride;
+#pragma unroll
+    for (int u = 0; u < kGatherMaxLoads; ++u) {
+      const int j = u * kGatherThreads + tid;
+      buf[u] = load16(v >= 0 && j < g.page_vecs ? src + (int64_t)j * 16 : g.q);
+    }
+  };
+  auto settle = [&](const u32x4 *buf, char *dst) {
+    if (dst == nullptr) return;
+#pragma unroll
+    for (int u = 0; u < kGatherMaxLoads; ++u) {
+      const int j = u * kGatherThreads + tid;
+      if (j < g.page_vecs) store16(dst + (int64_t)j * 16, buf[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kGatherMaxLoads; ++u) {
+      if (u * kGatherThreads >= g.page_vecs) continue;  // uniform
+      const bool tok = u * kGatherThreads + tid < g.page_vecs;
+      const u32x4 data = tok ? buf[u] : u32x4{0, 0, 0, 0};
+      float vf[V];
+      unpack<T>(data, vf);
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        const float sk = group_sum<kLanes>(dot16<T>(qv[r], data)) * g.scale_log2;
+        const float so = __shfl_xor(sk, kLanes, 64);  // a value lane takes its key lane's
+        float sc = is_v ? so : sk;
+        if (!tok) sc = -INFINITY;
+        const float mn = fmaxf(m[r], sc);
+        const float alpha = fast_exp2(m[r] - mn);
+        const float pw = fast_exp2(sc - mn);
+        m[r] = mn;
+        l[r] = l[r] * alpha + pw;
+#pragma unroll
+        for (int x = 0; x < V; ++x) acc[r][x] = acc[r][x] * alpha + pw * vf[x];
+      }
+    }
+  };
+
+  for (int batch0 = 0; batch0 < n_mine; batch0 += kGatherIdBatch) {
+    const int n_batch = n_mine - batch0 < kGatherIdBatch ? n_mine - batch0 : kGatherIdBatch;
+    __syncthreads();  // the previous batch is no longer read
+    for (int n = tid; n < n_batch; n += kGatherThreads) {
+      const int64_t i = (int64_t)block_x + (int64_t)(batch0 + n) * n_blocks;
+      sm_slot[n] = mslot[i];
+      sm_page[n] = mpage[i];
+    }
+    __syncthreads();
+    // two page buffers in turn: one is stored and attended while the other fills
+    u32x4 a_buf[kGatherMaxLoads], b_buf[kGatherMaxLoads];
+    char *a_dst = nullptr, *b_dst = nullptr;
+    fetch(0, n_batch, a_buf, a_dst);
+    for (int n = 0; n < n_batch; n += 2) {
+      fetch(n + 1, n_batch, b_buf, b_dst);
+      settle(a_buf, a_dst);
+      fetch(n + 2, n_batch, a_buf, a_dst);
+      settle(b_buf, b_dst);
+    }
+  }
+
+  // Merge the tokens of a wave (lanes of equal position within a token pair up).
+#pragma unroll
+  for (int off = kTokLanes; off < 64; off <<= 1) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const float mo = __shfl_xor(m[r], off, 64);
+      const float lo = __shfl_xor(l[r], off, 64);
+      const float mn = fmaxf(m[r], mo);
+      const float wa = fast_exp2(m[r] - mn), wb = fast_exp2(mo - mn);
+      l[r] = l[r] * wa + lo * wb;
+#pragma unroll
+      for (int x = 0; x < V; ++x) {
+        const float ao = __shfl_xor(acc[r][x], off, 64);
+        acc[r][x] = acc[r][x] * wa + ao * wb;
+      }
+      m[r] = mn;
+    }
+  }
+  // Merge the waves through LDS; the value lanes of a wave's first token hold its state.
+  __shared__ float sm_m[kWaves][kRows];
+  __shared__ float sm_l[kWaves][kRows];
+  __shared__ float sm_acc[kWaves][kRows][D];
+  if (is_v && lane < kTokLanes) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      if (c == 0) {
+        sm_m[wave][r] = m[r];
+        sm_l[wave][r] = l[r];
+      }
+#pragma unroll
+      for (int x = 0; x < V; ++x) sm_acc[wave][r][c * V + x] = acc[r][x];
+    }
+  }
+  __syncthreads();
+  const int chunk_id = g.chunk0 + block_x;
+  for (int item = tid; item < kRows * D; item += kGatherThreads) {
+    const int r = item / D, d = item % D;
+    if (r >= g.rep) continue;
+    float mn = sm_m[0][r];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mn = fmaxf(mn, sm_m[w][r]);
+    float lt = 0.f, at = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float wgt = fast_exp2(sm_m[w][r] - mn);
+      lt += sm_l[w][r] * wgt;
+      at += sm_acc[w][r][d] * wgt;
+    }
+    const int64_t slot = (int64_t)chunk_id * g.n_q_heads + (int64_t)h * g.rep + r;
+    g.part_acc[slot * D + d] = at;
+    if (d == 0) {
+      g.part_ml[slot * 2] = mn;
+      g.part_ml[slot * 2 + 1] = lt;
+    }
+  }
+}
+
+template <typename T, int kLanes, int kRows>
+__global__ void __launch_bounds__(kGatherThreads)
+pages_gather_attend_kernel(const GatherAttendArgs g) {
+  gather_attend_block<T, kLanes, kRows>(g, blockIdx.x, gridDim.x);
+}
+
+// Both of the above in one launch: blocks [0, g_blocks) of every kv head run the
+// page stream, the others the first attention pass (prefix minus the slots under
+// rewrite, plus the local segment).  One kernel instead of two on two streams
+// keeps the step a plain chain of launches: no fork and join around the long
+// pole of the step, each of which costs about 5 us of dependency latency.
+static_assert(kGatherThreads == kAttnThreads, "one block shape for both roles");
+template <typename T, int kLanes, int kRowsAttn, int kRowsGather>
+__global__ void __launch_bounds__(kAttnThreads)
+decode_stream_attend_kernel(const AttnArgs a, const GatherAttendArgs g, const int g_blocks) {
+  if ((int)blockIdx.x < g_blocks) {
+    if (blockIdx.z == 0) gather_attend_block<T, kLanes, kRowsGather>(g, blockIdx.x, g_blocks);
+  } else {
+    attention_split_block<T, kLanes, kRowsAttn, false>(a, (int)blockIdx.x - g_blocks);
+  }
+}
+
 // Merge the partials of one query head.  One 512-thread block per head.  The
 // softmax statistics are tiny, so every wave reduces them for itself (no
 // barrier); then a thread owns four adjacent output channels of every 16th
@@ -604,9 +828,31 @@ static void launch_split(AttnArgs a, int first_chunk, int n_launch, int n_kv_hea
 // merge.  Issued as two calls around a page stream, the first call also merges its own
 // chunks (into `out` and into one partial), so that the second call, the part
 // the step waits for, merges only that partial and the tail's.
+// The page stream and the first attention pass as one launch.
+template <typename T, int kLanes>
+static void launch_stream_attend(AttnArgs a, const GatherAttendArgs &g, int g_blocks, int n_chunks,
+                                 int n_kv_heads, hipStream_t s) {
+  a.chunk_base = 0;
+  const int rep = a.rep;
+  if (rep > 4 && kLanes <= 16) {
+    const dim3 grid(g_blocks + n_chunks, n_kv_heads, 1);
+    hipLaunchKernelGGL((decode_stream_attend_kernel<T, (kLanes <= 16 ? kLanes : 16), 8, 8>), grid,
+                       dim3(kAttnThreads), 0, s, a, g, g_blocks);
+  } else {
+    const dim3 grid(g_blocks + n_chunks, n_kv_heads, (unsigned)ceil_div(rep, 4));
+    if (rep > 4)
+      hipLaunchKernelGGL((decode_stream_attend_kernel<T, kLanes, 4, 8>), grid, dim3(kAttnThreads),
+                         0, s, a, g, g_blocks);
+    else
+      hipLaunchKernelGGL((decode_stream_attend_kernel<T, kLanes, 4, 4>), grid, dim3(kAttnThreads),
+                         0, s, a, g, g_blocks);
+  }
+}
+
 template <typename T>
 static int launch_attention(const AttnArgs &a, int phase, int n_kv_heads, int lanes, int head_dim,
-                            void *out, int64_t out_head_stride, float *lse_out, hipStream_t s) {
+                            void *out, int64_t out_head_stride, float *lse_out,
+                            const GatherAttendArgs *stream_args, hipStream_t s) {
 #define DA_ATTN_LAUNCH(tail, first, count)                                     \
   switch (lanes) {                                                             \
     case 4: launch_split<T, 4, tail>(a, first, count, n_kv_heads, s); break;   \
@@ -618,7 +864,17 @@ static int launch_attention(const AttnArgs &a, int phase, int n_kv_heads, int la
 #define DA_ATTN_MERGE(mode)                                                                    \
   hipLaunchKernelGGL(decode_attention_merge_kernel<T>, dim3(a.n_q_heads), dim3(kMergeThreads), \
                      0, s, a, mode, head_dim, (char *)out, out_head_stride, lse_out)
-  if (phase & DA_PHASE_FIRST) {
+  if (phase & DA_PHASE_STREAM) {
+    const int n_chunks = a.n_pchunks + a.n_lchunks;
+    switch (lanes) {
+      case 4: launch_stream_attend<T, 4>(a, *stream_args, a.gather_blocks, n_chunks, n_kv_heads, s); break;
+      case 8: launch_stream_attend<T, 8>(a, *stream_args, a.gather_blocks, n_chunks, n_kv_heads, s); break;
+      case 16: launch_stream_attend<T, 16>(a, *stream_args, a.gather_blocks, n_chunks, n_kv_heads, s); break;
+      case 32: launch_stream_attend<T, 32>(a, *stream_args, a.gather_blocks, n_chunks, n_kv_heads, s); break;
+    }
+    int rc = launch_status("da_decode_attention(page stream + first pass)");
+    if (rc) return rc;
+  } else if (phase & DA_PHASE_FIRST) {
     DA_ATTN_LAUNCH(false, 0, a.n_pchunks + a.n_lchunks)
     int rc = launch_status("da_decode_attention(split)");
     if (rc) return rc;
@@ -648,203 +904,6 @@ static int launch_attention(const AttnArgs &a, int phase, int n_kv_heads, int la
   return DA_OK;
 }
 
-
-// ---------------------------------------------------------------------------
-// Page stream with attention riding on it.  A block copies the pages of one kv
-// head's miss list (entries blockIdx.x, += gridDim.x) from the host page store
-// into their slots, 16 bytes per lane, and the registers the page passes
-// through also feed the attention of this step's query over that page: the
-// re-assigned slots then need no second pass after the stream has finished.
-// A page holds page_size tokens, each token its K row followed by its V row,
-// so 2*kLanes adjacent lanes hold one token: the lower kLanes its key (they
-// produce the score), the upper kLanes its value (they keep the softmax state
-// and the weighted sum).  The next page's loads are issued before the current
-// page is stored and attended, so the host link never waits for arithmetic.
-// Every block with an entry to copy leaves one partial (all query rows of the
-// kv head) at chunk id gather_chunk0 + blockIdx.x.
-struct GatherAttendArgs {
-  const char *dram;
-  int64_t dram_head_stride, dram_page_stride;
-  char *hbm;
-  int64_t hbm_head_stride, hbm_slot_stride;
-  int page_vecs;  // 16-byte lanes per page
-  const int32_t *miss_page, *miss_slot, *miss_count;
-  int K;
-  const char *q;
-  int64_t q_head_stride;
-  int rep, n_q_heads;
-  float scale_log2;
-  float *part_ml, *part_acc;
-  int chunk0;
-};
-
-constexpr int kGatherThreads = 256;
-constexpr int kGatherMaxLoads = 4;  // 16-byte loads per lane and page: pages up to 16 KiB
-constexpr int kGatherIdBatch = 1024;  // miss-list entries of a block staged in LDS at a time
-
-template <typename T, int kLanes, int kRows>
-__global__ void __launch_bounds__(kGatherThreads)
-pages_gather_attend_kernel(const GatherAttendArgs g) {
-  constexpr int V = T::kVec;
-  constexpr int D = kLanes * V;
-  constexpr int kTokLanes = 2 * kLanes;
-  constexpr int kWaves = kGatherThreads / 64;
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int within = tid % kTokLanes;
-  const bool is_v = within >= kLanes;
-  const int c = within % kLanes;
-  const int h = blockIdx.y;
-  const int n_miss = g.miss_count[h];
-  if ((int)blockIdx.x >= n_miss) return;  // the merge does not count this block either
-
-  u32x4 qv[kRows];
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const int rr = r < g.rep ? r : g.rep - 1;
-    qv[r] = load16(g.q + ((int64_t)(h * g.rep + rr) * g.q_head_stride) * T::kBytes + c * 16);
-  }
-  float m[kRows], l[kRows], acc[kRows][V];
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    m[r] = kMinusHuge;
-    l[r] = 0.f;
-#pragma unroll
-    for (int i = 0; i < V; ++i) acc[r][i] = 0.f;
-  }
-
-  const int32_t *mpage = g.miss_page + (int64_t)h * g.K;
-  const int32_t *mslot = g.miss_slot + (int64_t)h * g.K;
-  // This block's entries (slot, page), staged in LDS a batch at a time: a page's
-  // loads then depend on no other global load, and the next page is always in
-  // flight while the current one is stored and attended.
-  __shared__ int32_t sm_slot[kGatherIdBatch], sm_page[kGatherIdBatch];
-  const int n_mine = (n_miss - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-  // Issues the loads of this block's n-th staged entry; dst == nullptr marks a
-  // superseded one.  Always kGatherMaxLoads loads per lane, lanes with nothing to
-  // fetch reading the query instead: with a fixed count the wait for one page's
-  // data can leave the next page's loads outstanding.
-  auto fetch = [&](int n, int n_batch, u32x4 *buf, char *&dst) {
-    const bool real = n < n_batch;  // past the batch: the same loads, all of them idle
-    const int32_t v = real ? sm_slot[n] : -1;
-    const int32_t p = real ? sm_page[n] : 0;
-    const char *src = g.dram + h * g.dram_head_stride + p * g.dram_page_stride;
-    dst = v < 0 ? nullptr : g.hbm + h * g.hbm_head_stride + v * g.hbm_slot_stride;
-#pragma unroll
-    for (int u = 0; u < kGatherMaxLoads; ++u) {
-      const int j = u * kGatherThreads + tid;
-      buf[u] = load16(v >= 0 && j < g.page_vecs ? src + (int64_t)j * 16 : g.q);
-    }
-  };
-  auto settle = [&](const u32x4 *buf, char *dst) {
-    if (dst == nullptr) return;
-#pragma unroll
-    for (int u = 0; u < kGatherMaxLoads; ++u) {
-      const int j = u * kGatherThreads + tid;
-      if (j < g.page_vecs) store16(dst + (int64_t)j * 16, buf[u]);
-    }
-#pragma unroll
-    for (int u = 0; u < kGatherMaxLoads; ++u) {
-      if (u * kGatherThreads >= g.page_vecs) continue;  // uniform
-      const bool tok = u * kGatherThreads + tid < g.page_vecs;
-      const u32x4 data = tok ? buf[u] : u32x4{0, 0, 0, 0};
-      float vf[V];
-      unpack<T>(data, vf);
-#pragma unroll
-      for (int r = 0; r < kRows; ++r) {
-        const float sk = group_sum<kLanes>(dot16<T>(qv[r], data)) * g.scale_log2;
-        const float so = __shfl_xor(sk, kLanes, 64);  // a value lane takes its key lane's
-        float sc = is_v ? so : sk;
-        if (!tok) sc = -INFINITY;
-        const float mn = fmaxf(m[r], sc);
-        const float alpha = fast_exp2(m[r] - mn);
-        const float pw = fast_exp2(sc - mn);
-        m[r] = mn;
-        l[r] = l[r] * alpha + pw;
-#pragma unroll
-        for (int x = 0; x < V; ++x) acc[r][x] = acc[r][x] * alpha + pw * vf[x];
-      }
-    }
-  };
-
-  for (int batch0 = 0; batch0 < n_mine; batch0 += kGatherIdBatch) {
-    const int n_batch = n_mine - batch0 < kGatherIdBatch ? n_mine - batch0 : kGatherIdBatch;
-    __syncthreads();  // the previous batch is no longer read
-    for (int n = tid; n < n_batch; n += kGatherThreads) {
-      const int64_t i = (int64_t)blockIdx.x + (int64_t)(batch0 + n) * gridDim.x;
-      sm_slot[n] = mslot[i];
-      sm_page[n] = mpage[i];
-    }
-    __syncthreads();
-    // two page buffers in turn: one is stored and attended while the other fills
-    u32x4 a_buf[kGatherMaxLoads], b_buf[kGatherMaxLoads];
-    char *a_dst = nullptr, *b_dst = nullptr;
-    fetch(0, n_batch, a_buf, a_dst);
-    for (int n = 0; n < n_batch; n += 2) {
-      fetch(n + 1, n_batch, b_buf, b_dst);
-      settle(a_buf, a_dst);
-      fetch(n + 2, n_batch, a_buf, a_dst);
-      settle(b_buf, b_dst);
-    }
-  }
-
-  // Merge the tokens of a wave (lanes of equal position within a token pair up).
-#pragma unroll
-  for (int off = kTokLanes; off < 64; off <<= 1) {
-#pragma unroll
-    for (int r = 0; r < kRows; ++r) {
-      const float mo = __shfl_xor(m[r], off, 64);
-      const float lo = __shfl_xor(l[r], off, 64);
-      const float mn = fmaxf(m[r], mo);
-      const float wa = fast_exp2(m[r] - mn), wb = fast_exp2(mo - mn);
-      l[r] = l[r] * wa + lo * wb;
-#pragma unroll
-      for (int x = 0; x < V; ++x) {
-        const float ao = __shfl_xor(acc[r][x], off, 64);
-        acc[r][x] = acc[r][x] * wa + ao * wb;
-      }
-      m[r] = mn;
-    }
-  }
-  // Merge the waves through LDS; the value lanes of a wave's first token hold its state.
-  __shared__ float sm_m[kWaves][kRows];
-  __shared__ float sm_l[kWaves][kRows];
-  __shared__ float sm_acc[kWaves][kRows][D];
-  if (is_v && lane < kTokLanes) {
-#pragma unroll
-    for (int r = 0; r < kRows; ++r) {
-      if (c == 0) {
-        sm_m[wave][r] = m[r];
-        sm_l[wave][r] = l[r];
-      }
-#pragma unroll
-      for (int x = 0; x < V; ++x) sm_acc[wave][r][c * V + x] = acc[r][x];
-    }
-  }
-  __syncthreads();
-  const int chunk_id = g.chunk0 + blockIdx.x;
-  for (int item = tid; item < kRows * D; item += kGatherThreads) {
-    const int r = item / D, d = item % D;
-    if (r >= g.rep) continue;
-    float mn = sm_m[0][r];
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w) mn = fmaxf(mn, sm_m[w][r]);
-    float lt = 0.f, at = 0.f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      const float wgt = fast_exp2(sm_m[w][r] - mn);
-      lt += sm_l[w][r] * wgt;
-      at += sm_acc[w][r][d] * wgt;
-    }
-    const int64_t slot = (int64_t)chunk_id * g.n_q_heads + (int64_t)h * g.rep + r;
-    g.part_acc[slot * D + d] = at;
-    if (d == 0) {
-      g.part_ml[slot * 2] = mn;
-      g.part_ml[slot * 2 + 1] = lt;
-    }
-  }
-}
 
 template <typename T, int kLanes>
 static void launch_gather_attend(const GatherAttendArgs &g, dim3 grid, hipStream_t s) {
@@ -1018,8 +1077,11 @@ extern "C" int da_decode_attention_paged(
     DA_REQUIRE(overlap->slot_epoch && overlap->epoch && overlap->miss_slot &&
                    overlap->miss_count && overlap->miss_capacity >= 0,
                "da_decode_attention: incomplete overlap description");
-    DA_REQUIRE(overlap->phase >= 1 && overlap->phase <= 7, "da_decode_attention: bad phase %d",
+    DA_REQUIRE(overlap->phase >= 1 && overlap->phase <= 15, "da_decode_attention: bad phase %d",
                overlap->phase);
+    DA_REQUIRE(!(overlap->phase & DA_PHASE_STREAM) ||
+                   ((overlap->phase & DA_PHASE_FIRST) && overlap->gather_blocks >= 1),
+               "da_decode_attention: DA_PHASE_STREAM goes with DA_PHASE_FIRST and gather_blocks >= 1");
     a.page_size = overlap->page_size;
     a.page_shift = -1;
     for (int b = 0; b < 31; ++b)
@@ -1055,16 +1117,52 @@ extern "C" int da_decode_attention_paged(
   a.part_ml = a.part_acc + (size_t)p.total() * n_q_heads * head_dim;
   hipStream_t s = (hipStream_t)stream;
   if (p.n_p + p.n_l == 0) return fail(DA_EINVAL, "da_decode_attention: no key/value rows at all");
+  GatherAttendArgs g = {};
+  if (phase & DA_PHASE_STREAM) {
+    const int64_t page_vecs = (int64_t)overlap->page_size * 2 * lanes;
+    if (lanes > 32 || a.rep > 8 || page_vecs > kGatherThreads * kGatherMaxLoads)
+      return fail(DA_ENOTSUP,
+                  "da_decode_attention: DA_PHASE_STREAM needs rows of 64..512 bytes, at most 8 query "
+                  "heads per kv head and pages up to %d bytes",
+                  kGatherThreads * kGatherMaxLoads * 16);
+    DA_REQUIRE(overlap->dram && overlap->hbm && overlap->miss_page,
+               "da_decode_attention: DA_PHASE_STREAM without the page stream's operands");
+    DA_REQUIRE(overlap->dram_head_stride_bytes % 16 == 0 &&
+                   overlap->dram_page_stride_bytes % 16 == 0 &&
+                   overlap->hbm_head_stride_bytes % 16 == 0 &&
+                   overlap->hbm_slot_stride_bytes % 16 == 0 && (uintptr_t)overlap->dram % 16 == 0 &&
+                   (uintptr_t)overlap->hbm % 16 == 0,
+               "da_decode_attention: page stores must be 16-byte aligned");
+    g.dram = (const char *)overlap->dram;
+    g.dram_head_stride = overlap->dram_head_stride_bytes;
+    g.dram_page_stride = overlap->dram_page_stride_bytes;
+    g.hbm = (char *)overlap->hbm;
+    g.hbm_head_stride = overlap->hbm_head_stride_bytes;
+    g.hbm_slot_stride = overlap->hbm_slot_stride_bytes;
+    g.page_vecs = (int)page_vecs;
+    g.miss_page = overlap->miss_page;
+    g.miss_slot = overlap->miss_slot;
+    g.miss_count = overlap->miss_count;
+    g.K = overlap->miss_capacity;
+    g.q = a.q;
+    g.q_head_stride = q_head_stride;
+    g.rep = a.rep;
+    g.n_q_heads = n_q_heads;
+    g.scale_log2 = a.scale_log2;
+    g.part_acc = a.part_acc;
+    g.part_ml = a.part_ml;
+    g.chunk0 = a.gather_chunk0;
+  }
   switch (dtype) {
     case DA_F32:
       return launch_attention<F32>(a, phase, n_kv_heads, lanes, head_dim, out, out_head_stride,
-                                   lse_out, s);
+                                   lse_out, &g, s);
     case DA_F16:
       return launch_attention<F16>(a, phase, n_kv_heads, lanes, head_dim, out, out_head_stride,
-                                   lse_out, s);
+                                   lse_out, &g, s);
     default:
       return launch_attention<BF16>(a, phase, n_kv_heads, lanes, head_dim, out, out_head_stride,
-                                    lse_out, s);
+                                    lse_out, &g, s);
   }
 }
 

@@ -27,27 +27,40 @@ class PagedPrefix:
     FIRST attends over the local window and every slot that keeps its page,
     FIRST_MERGE folds those partial results into one (both may run next to the
     stream), SECOND (after the stream has finished) attends over the re-assigned
-    slots and writes the output; FIRST | SECOND does everything at once."""
+    slots and writes the output; FIRST | SECOND does everything at once.  With
+    STREAM the page stream itself runs inside the launch of the FIRST pass."""
 
-    FIRST, SECOND, FIRST_MERGE = 1, 2, 4
+    FIRST, SECOND, FIRST_MERGE, STREAM = 1, 2, 4, 8
 
     def __init__(self, page_size: int, scratch, current_step: torch.Tensor, phase: int,
-                 gather_blocks: int = 0):
+                 gather_blocks: int = 0, page_stores=None):
         self.page_size = page_size
         self.scratch = scratch
         self.current_step = current_step
         self.phase = phase
-        # blocks per kv head of a pages_gather_attend stream that already covered
-        # the re-assigned slots (0: the SECOND pass attends over them)
+        # blocks per kv head of a page stream that attends over the pages it moves
+        # (0: the SECOND pass attends over the re-assigned slots)
         self.gather_blocks = gather_blocks
+        # STREAM: (dram_kv_cache, its device-visible address, hbm_kv_cache); the page
+        # stream then runs inside the launch of the FIRST pass
+        self.page_stores = page_stores
 
     def as_struct(self) -> "_lib.PagedOverlap":
         s = self.scratch
-        return _lib.PagedOverlap(
+        o = _lib.PagedOverlap(
             page_size=self.page_size, phase=self.phase, slot_epoch=s.slot_epoch.data_ptr(),
             slot_epoch_head_stride=s.slot_epoch.stride(0), epoch=self.current_step.data_ptr(),
             miss_slot=s.miss_slot.data_ptr(), miss_count=s.miss_count.data_ptr(),
             miss_capacity=s.miss_slot.shape[1], gather_blocks=self.gather_blocks)
+        if self.phase & self.STREAM:
+            dram, dram_ptr, hbm = self.page_stores
+            esz = dram.element_size()
+            o.dram, o.hbm, o.miss_page = dram_ptr, hbm.data_ptr(), s.miss_page.data_ptr()
+            o.dram_head_stride_bytes = dram.stride(0) * esz
+            o.dram_page_stride_bytes = dram.stride(1) * esz
+            o.hbm_head_stride_bytes = hbm.stride(0) * esz
+            o.hbm_slot_stride_bytes = hbm.stride(1) * esz
+        return o
 
 
 def attention_workspace(Hq: int, Hkv: int, D: int, dtype: torch.dtype, p_len: int, capacity: int,
@@ -204,7 +217,7 @@ class DRAMAttention(torch.nn.Module):
         self.register_buffer("cache_v", torch.zeros(cache_shape, device=device, dtype=dtype))
         self._workspace = None
         self._side_stream = None
-        # stream missed pages on a side stream underneath the attention pass
+        # run the page stream and the first attention pass concurrently (two streams)
         self.overlap_page_stream = True
         # attend over the streamed pages inside the page stream itself (when the
         # shape allows) instead of a pass over them after the stream
@@ -307,9 +320,20 @@ class DRAMAttention(torch.nn.Module):
         P = PagedPrefix
         if not self.overlap_page_stream:
             stream_pages()
-            # the same kernels as the overlapped order, so the same bits
-            attend(P.FIRST | P.FIRST_MERGE | P.SECOND)
+            # the same kernels as the concurrent order, so the same bits
+            attend((P.FIRST | P.SECOND) if fused else (P.FIRST | P.FIRST_MERGE | P.SECOND))
             return out
+        if fused:
+            # page stream and first attention pass in one launch, then the merge: the
+            # step stays a plain chain of launches on the caller's stream
+            decode_attention(*args, workspace=self._workspace, out=out[0, 0],
+                             cache_len_offset=offset,
+                             paged=PagedPrefix(self.page_size, scratch, lru.current_step,
+                                               P.STREAM | P.FIRST | P.SECOND, blocks,
+                                               lru.page_stores()))
+            return out
+        # Shapes the fused stream does not take: pages stream in on a side stream
+        # next to the first pass, and a tail pass covers them after the join.
         main = torch.cuda.current_stream(xq.device)
         if self._side_stream is None:
             self._side_stream = torch.cuda.Stream(device=xq.device)

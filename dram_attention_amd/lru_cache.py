@@ -191,6 +191,13 @@ class LRUCache(torch.nn.Module):
                             self.page_size, xq, scale, self.num_hbm_pages * self.page_size,
                             c_capacity, workspace, blocks_per_head, self._dram_device_ptr)
 
+    def page_stores(self):
+        """(dram_kv_cache, its device-visible address, hbm_kv_cache) for a page stream
+        that runs inside an attention launch."""
+        if self._dram_device_ptr is None:
+            self._dram_device_ptr = _lib.device_visible_ptr(self.dram_kv_cache)
+        return self.dram_kv_cache, self._dram_device_ptr, self.hbm_kv_cache
+
     def views(self) -> CacheOutput:
         return self._views()
 

@@ -221,7 +221,14 @@ int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
  * When the page stream of the step was da_pages_gather_attend, which attends
  * over the re-assigned slots itself, set `gather_blocks` to its
  * blocks_per_head: DA_PHASE_SECOND is then only the final merge.
- * The usual step: FIRST | FIRST_MERGE next to the stream, SECOND after the join.
+ *   DA_PHASE_STREAM      : together with DA_PHASE_FIRST: the page stream itself
+ *                          (the work of da_pages_gather_attend, with
+ *                          `gather_blocks` workgroups per kv head) runs inside
+ *                          the launch of the first pass, no second stream
+ *                          needed.  STREAM | FIRST | SECOND is a whole step in
+ *                          two launches.  Same shape limits as
+ *                          da_pages_gather_attend (DA_ENOTSUP otherwise).
+ * With two streams: FIRST | FIRST_MERGE next to the page stream, SECOND after the join.
  * FIRST | SECOND in one call (the page stream already complete) needs no
  * FIRST_MERGE.
  * The calls of a step must be given identical arguments otherwise.  The
@@ -230,6 +237,7 @@ int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
 #define DA_PHASE_FIRST 1
 #define DA_PHASE_SECOND 2
 #define DA_PHASE_FIRST_MERGE 4
+#define DA_PHASE_STREAM 8
 
 typedef struct da_paged_overlap {
   int32_t page_size;              /* tokens per slot; p_len = slots * page_size */
@@ -241,6 +249,12 @@ typedef struct da_paged_overlap {
   const int32_t *miss_count;      /* (Hkv) */
   int32_t miss_capacity;
   int32_t gather_blocks;          /* blocks_per_head of da_pages_gather_attend, else 0 */
+  /* DA_PHASE_STREAM only: the operands of the page stream, as da_pages_gather_attend takes them */
+  const void *dram;
+  int64_t dram_head_stride_bytes, dram_page_stride_bytes;
+  void *hbm;
+  int64_t hbm_head_stride_bytes, hbm_slot_stride_bytes;
+  const int32_t *miss_page;       /* (Hkv, miss_capacity) */
 } da_paged_overlap;
 
 int da_decode_attention_paged(const void *q, int64_t q_head_stride, int n_q_heads,
