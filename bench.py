@@ -8,8 +8,9 @@ top-k, LRU update, streaming of missed pages from pinned host DRAM, and decode
 attention over the resident pages + local window + new token.  Inputs of all
 steps are staged in HBM before the clock starts.  By default the step is
 captured once into a HIP graph (position and LRU step live on the device) and
-replayed; --eager issues the launches from Python every step; --no-overlap
-keeps the page stream and attention on one stream.
+replayed (--steps-per-graph consecutive steps per graph, as a model step of
+several layers would be); --eager issues the launches from Python every step;
+--no-overlap runs the page stream to completion before attention starts.
 
 Prints ONE JSON line: the BASELINE metric plus `roofline` (the dominant HBM
 kernel, timed live with events on the launch stream) and `cpu_baseline` (the CPU
@@ -41,6 +42,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="128k", choices=sorted(WORKLOAD_INDEX))
     ap.add_argument("--eager", action="store_true", help="no HIP graph: launch from Python each step")
+    ap.add_argument("--steps-per-graph", type=int, default=8,
+                    help="decode steps captured into one HIP graph (the reference's example "
+                         "captures a whole model step, i.e. 32 attention layers, per graph)")
     ap.add_argument("--no-overlap", action="store_true",
                     help="page stream and attention serialised on one stream")
     ap.add_argument("--seed", type=int, default=0)
@@ -254,7 +258,7 @@ def main():
     torch.cuda.synchronize()
 
     # -- warm-up (also resolves the pinned-host device address before any capture)
-    graph = None
+    graph, graph_many, spg = None, None, 1
     if args.eager:
         for _ in range(args.warmup):
             layer.step_from_device_state()
@@ -269,15 +273,23 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             layer.step_from_device_state()
-        # the capture itself executed nothing; replay for the remaining warm-up steps
+        spg = max(1, min(args.steps_per_graph, args.steps))
+        if spg > 1:
+            graph_many = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph_many):
+                for _ in range(spg):
+                    layer.step_from_device_state()
+        # the captures themselves executed nothing; replay for the remaining warm-up steps
         for _ in range(max(args.warmup - 2, 0)):
             graph.replay()
     torch.cuda.synchronize()
 
-    # -- timed region
+    # -- timed region: exactly args.steps decode steps
     t0 = time.perf_counter()
     if graph is not None:
-        for _ in range(args.steps):
+        for _ in range(args.steps // spg if graph_many is not None else 0):
+            graph_many.replay()
+        for _ in range(args.steps % spg if graph_many is not None else args.steps):
             graph.replay()
     else:
         for _ in range(args.steps):
@@ -327,7 +339,7 @@ def main():
                         f"1 layer, {w.n_q_heads}q/{w.n_kv_heads}kv heads, D {w.head_dim}, "
                         f"{w.dram_tokens}-token prefix in pinned host DRAM ({w.n_dram_pages} pages/head), "
                         f"local {w.local_cache}, LRU {w.lru_tokens} tokens, top-k {w.top_k_tokens} tokens",
-            "launch": "eager" if args.eager else "hip-graph replay",
+            "launch": "eager" if args.eager else f"hip-graph replay, {spg} decode steps per graph",
             "page_stream": "serialised" if args.no_overlap else "in the launch of the first attention pass",
             "seed": args.seed,
         },
