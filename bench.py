@@ -243,6 +243,10 @@ def main():
         print("bench.py measures one GPU: this hot path is a single-device decode step "
               "(run with --gpus 1)", file=sys.stderr)
         return 2
+    if args.profile_steps <= 0:
+        print("bench.py: --profile-steps must be at least 1 (the roofline figures come from that pass)",
+              file=sys.stderr)
+        return 2
     if not torch.cuda.is_available():
         print("bench.py needs a GPU: the HIP kernels are the only implementation", file=sys.stderr)
         return 2
@@ -320,7 +324,7 @@ def main():
     # HBM bytes per launch of the roofline kernel from the committed counter runs
     # (profiles/bench_128k_hbm_traffic_pmc.md: FETCH_SIZE x 2.0 + WRITE_SIZE); only
     # known for the workload those runs used
-    traffic = 154.7e6 if w.name == "128k" else None
+    traffic = 152.5e6 if w.name == "128k" else None
     result = {
         "metric": "decode steps/sec per layer at 128K ctx; scorer+attn HBM GB/s vs peak",
         "value": args.steps / dt,
