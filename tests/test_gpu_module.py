@@ -210,6 +210,27 @@ def test_decode_parity_device_side_position_and_rep8():
     run_parity(w, 2, w.steps, atol=2e-2, rtol=1e-2, device_pos=True)
 
 
+def test_decode_parity_more_requests_than_slots():
+    """rep * pages-per-head > slots: the LRU takes the serial walk, victims wrap
+    onto slots handed out earlier in the same step, and the superseded entries of
+    the miss list must be skipped by the page stream and by its attention."""
+    w = WORKLOADS["128k"].scaled(dram_tokens=8192, local_cache=512, lru_tokens=1024,
+                                 top_k_tokens=512, steps=5)
+    assert w.rep * w.pages_per_q_head > w.n_hbm_pages
+    run_parity(w, 3, w.steps, atol=2e-2, rtol=1e-2)
+
+
+def test_decode_parity_wide_gqa_group_takes_the_tail_pass():
+    """16 query heads per kv head: outside what the attending page stream takes, so
+    pages stream in on a side stream and a tail pass covers them."""
+    from dram_attention_amd.lru_kernel import gather_attend_supported
+
+    w = WORKLOADS["128k"].scaled(n_q_heads=32, n_kv_heads=2, dram_tokens=8192, local_cache=512,
+                                 lru_tokens=2048, top_k_tokens=128, steps=4)
+    assert not gather_attend_supported(w.n_q_heads, w.n_kv_heads, w.head_dim, w.page_size, w.dtype)
+    run_parity(w, 5, w.steps, atol=2e-2, rtol=1e-2)
+
+
 def test_page_stream_overlap_changes_nothing():
     """Attention issued around a concurrent page stream (two phases, side stream)
     gives the bits of the serialised order, and both agree with one plain pass."""
