@@ -279,7 +279,7 @@ extern "C" size_t da_lru_update_workspace_bytes(int, int, int64_t, int) { return
 
 extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_itype,
                              int n_kv_heads, int k, int64_t n_dram_pages, int n_hbm_pages,
-                             int32_t *step, int bump_step, void *access_time,
+                             int32_t *step, int flags, void *access_time,
                              int64_t time_head_stride, int time_type, void *d2h,
                              int64_t d2h_head_stride, void *h2d, int64_t h2d_head_stride,
                              int map_itype, uint8_t *hit_mask, int32_t *miss_page,
@@ -301,7 +301,9 @@ extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_i
              "da_lru_update: workspace too small");
   DA_REQUIRE(n_hbm_pages > 0 || k == 0, "da_lru_update: no HBM slots");
   DA_REQUIRE(n_dram_pages <= 0x7fffffff, "da_lru_update: page ids must fit int32");
-  const int serial = (k > n_hbm_pages || k > kLruMaxK) ? 1 : 0;
+  DA_REQUIRE((flags & ~(DA_LRU_BUMP_STEP | DA_LRU_SERIAL_WALK)) == 0, "da_lru_update: unknown flags %d", flags);
+  const int bump_step = (flags & DA_LRU_BUMP_STEP) ? 1 : 0;
+  const int serial = ((flags & DA_LRU_SERIAL_WALK) || k > n_hbm_pages || k > kLruMaxK) ? 1 : 0;
   if (serial && n_hbm_pages > kSelMaxK)
     return fail(DA_ENOTSUP,
                 "da_lru_update: k %d > slots %d needs the serial walk, which orders at most %d "

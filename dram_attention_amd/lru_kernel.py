@@ -48,9 +48,11 @@ def lru_update(
     hbm_kv_cache: torch.Tensor,
     scratch: LruScratch,
     bump_step: bool,
+    serial_walk: bool = False,
 ) -> None:
     """The metadata half of a step: touch, evict, assign; leaves the miss list in
-    ``scratch`` (one launch on the current stream)."""
+    ``scratch`` (one launch on the current stream).  ``serial_walk`` forces the
+    literal one-request-at-a-time walk (same result, for checks and baselines)."""
     num_heads, num_dram_pages, page_dim = dram_kv_cache.shape
     _, k = topk_dram_page_index.shape
     assert (
@@ -82,7 +84,7 @@ def lru_update(
         lib.da_lru_update(
             topk_dram_page_index.data_ptr(), topk_dram_page_index.stride(0),
             _lib.itype_code(topk_dram_page_index.dtype), num_heads, k, num_dram_pages,
-            num_hbm_pages, current_step.data_ptr(), int(bump_step),
+            num_hbm_pages, current_step.data_ptr(), int(bump_step) | (2 if serial_walk else 0),
             page_access_time.data_ptr(), page_access_time.stride(0),
             _lib.time_code(page_access_time.dtype),
             dram_page_to_hbm_page_mapping.data_ptr(), dram_page_to_hbm_page_mapping.stride(0),
@@ -170,11 +172,12 @@ def lru_update_and_gather(
     scratch: LruScratch,
     bump_step: bool,
     dram_device_ptr: Optional[int] = None,
+    serial_walk: bool = False,
 ) -> None:
     """Two launches on the current stream: metadata update, then page gather."""
     lru_update(dram_kv_cache, page_access_time, dram_page_to_hbm_page_mapping,
                hbm_page_to_dram_page_mapping, topk_dram_page_index, current_step, hbm_kv_cache,
-               scratch, bump_step)
+               scratch, bump_step, serial_walk)
     pages_gather(dram_kv_cache, hbm_kv_cache, scratch, topk_dram_page_index.shape[1],
                  dram_device_ptr)
 

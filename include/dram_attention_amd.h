@@ -115,9 +115,9 @@ int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
  * Replaces _update_page_access_time_, torch.argsort(page_access_time,
  * stable=True) and the metadata half of _load_lru_cache_inline_kernel in
  * dram_attention/lru_triton_kernel.py:6-194 (and current_step.add_(1),
- * dram_attention/lru_cache.py:224, when `bump_step` is set).
+ * dram_attention/lru_cache.py:224, when DA_LRU_BUMP_STEP is set in `flags`).
  *   idx          : (Hkv, K) requested DRAM pages in visiting order (itype idx_itype)
- *   step         : one int32; with bump_step the kernel uses *step+1 and stores it
+ *   step         : one int32; with DA_LRU_BUMP_STEP the kernel uses *step+1 and stores it
  *   access_time  : (Hkv, N_hbm) last-use step per slot (fp32 or int32)
  *   d2h          : (Hkv, P) slot of each DRAM page or -1;  h2d : (Hkv, N_hbm) page per slot
  *                  (both of itype map_itype); updated in place
@@ -129,16 +129,21 @@ int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
  *                  the page stream of this step is (still) writing
  * The end state equals the reference's serial walk for every input; K <=
  * N_hbm runs fully parallel, K > N_hbm falls back to one serial lane per head.
+ * DA_LRU_SERIAL_WALK in `flags` takes that literal walk for any K (a checking
+ * and benchmarking aid: the result is the same, only slower).
  * A miss_slot of -1 marks an entry whose slot was re-assigned later in the
  * same call (possible only when K > N_hbm); da_pages_gather skips it.
  * workspace: da_lru_update_workspace_bytes(...) bytes, ZEROED ONCE by the
  * caller before the first call and left alone afterwards.
  */
+#define DA_LRU_BUMP_STEP 1
+#define DA_LRU_SERIAL_WALK 2
+
 size_t da_lru_update_workspace_bytes(int n_kv_heads, int k, int64_t n_dram_pages,
                                      int n_hbm_pages);
 int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_itype,
                   int n_kv_heads, int k, int64_t n_dram_pages, int n_hbm_pages,
-                  int32_t *step, int bump_step, void *access_time,
+                  int32_t *step, int flags, void *access_time,
                   int64_t time_head_stride, int time_type, void *d2h,
                   int64_t d2h_head_stride, void *h2d, int64_t h2d_head_stride,
                   int map_itype, uint8_t *hit_mask, int32_t *miss_page,

@@ -201,7 +201,7 @@ def test_load_lru_cache_reference_kats(name):
 
 
 def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat16, page_dim=256,
-              hot=None):
+              hot=None, serial_walk=False):
     """Random request trace on LRUCache-like state; compares every buffer with the
     oracle's serial walk after every step."""
     from dram_attention_amd.lru_kernel import LruScratch, lru_update_and_gather
@@ -226,7 +226,7 @@ def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat1
             idx = rng.integers(0, P, (H, K))
         hit_o, miss_o = O.lru_load(st, idx, s, as_np(dram), as_np(hbm_o))
         lru_update_and_gather(dram_dev, time, d2h, h2d, torch.from_numpy(idx).to(itype).to(DEV),
-                              step, hbm, scratch, bump_step=True)
+                              step, hbm, scratch, bump_step=True, serial_walk=serial_walk)
         torch.cuda.synchronize()
         assert step.item() == s
         assert np.array_equal(time.cpu().numpy().astype(np.float32), st.time), f"time, step {s}"
@@ -259,6 +259,12 @@ def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat1
 def test_lru_update_matches_serial_walk(H, P, N, K, itype, ttype, pinned):
     lru_trace(H, P, N, K, 12, 100 + K, itype, ttype, pinned)
     lru_trace(H, P, N, K, 12, 200 + K, itype, ttype, pinned, hot=max(2, P // 8))
+
+
+def test_lru_update_forced_serial_walk_gives_the_same_state():
+    """The literal walk, forced where the parallel form applies: same end state."""
+    lru_trace(4, 1024, 256, 200, 10, 77, torch.int64, torch.float32, False, serial_walk=True)
+    lru_trace(2, 512, 128, 128, 6, 78, torch.int32, torch.int32, True, hot=64, serial_walk=True)
 
 
 @pytest.mark.parametrize("H,P,N,K", [(2, 40, 6, 17), (1, 8, 2, 3), (3, 200, 50, 120)])
