@@ -47,8 +47,12 @@ def parse_args():
                          "captures a whole model step, i.e. 32 attention layers, per graph)")
     ap.add_argument("--no-overlap", action="store_true",
                     help="page stream and attention serialised on one stream")
+    ap.add_argument("--layers", type=int, default=1,
+                    help="attention layers per model step, each with its own page cache and inputs "
+                         "(seed + layer); 32 with workload 128k is configs[3].  One model step per "
+                         "graph; value stays per layer: layer-steps per second")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--cpu-steps", type=int, default=8, help="steps of the CPU oracle to time (0 = skip)")
+    ap.add_argument("--cpu-steps", type=int, default=64, help="steps of the CPU oracle to time (0 = skip)")
     ap.add_argument("--reference-shaped-steps", type=int, default=24,
                     help="steps of the reference-shaped stand-in pipeline to time (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=16, help="extra steps timed per kernel with events")
@@ -368,31 +372,44 @@ def main():
     torch.cuda.set_device(dev)
     w = WORKLOADS[args.workload]
     total = args.warmup + args.steps + args.profile_steps + 4
-    layer = Layer(w, args.seed, total, dev, overlap=not args.no_overlap)
+    layers = []
+    for li in range(max(args.layers, 1)):
+        layers.append(Layer(w, args.seed + li, total, dev, overlap=not args.no_overlap))
+        if li > 0:
+            layers[-1].prompt = None   # only layer 0 feeds the CPU baseline
+        if args.layers > 1:
+            print(f"bench.py: layer {li + 1}/{args.layers} built", file=sys.stderr, flush=True)
+    layer = layers[0]
+    n_layers = len(layers)
+
+    def model_step():
+        for l_ in layers:
+            l_.step_from_device_state()
+
     torch.cuda.synchronize()
 
     # -- warm-up (also resolves the pinned-host device address before any capture)
     graph, graph_many, spg = None, None, 1
     if args.eager:
         for _ in range(args.warmup):
-            layer.step_from_device_state()
+            model_step()
     else:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             for _ in range(2):
-                layer.step_from_device_state()
+                model_step()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            layer.step_from_device_state()
-        spg = max(1, min(args.steps_per_graph, args.steps))
+            model_step()
+        spg = max(1, min(args.steps_per_graph, args.steps)) if n_layers == 1 else 1
         if spg > 1:
             graph_many = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph_many):
                 for _ in range(spg):
-                    layer.step_from_device_state()
+                    model_step()
         # the captures themselves executed nothing; replay for the remaining warm-up steps
         for _ in range(max(args.warmup - 2, 0)):
             graph.replay()
@@ -407,10 +424,10 @@ def main():
             graph.replay()
     else:
         for _ in range(args.steps):
-            layer.step_from_device_state()
+            model_step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
+    ms_per_step = dt / (args.steps * n_layers) * 1e3
 
     # -- per-kernel pass and traffic counters
     kernel_us, miss_per_step, local_rows = time_kernels(layer, args.profile_steps)
@@ -437,7 +454,7 @@ def main():
     traffic = 152.5e6 if w.name == "128k" else None
     result = {
         "metric": "decode steps/sec per layer at 128K ctx; scorer+attn HBM GB/s vs peak",
-        "value": args.steps / dt,
+        "value": args.steps * n_layers / dt,
         "unit": "decode steps/s per layer",
         "n_gpus": 1,
         "steps": args.steps,
@@ -449,11 +466,14 @@ def main():
         "dtype": {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[w.dtype],
         "data": "synthetic",
         "config": {
-            "workload": f"configs[{WORKLOAD_INDEX[w.name]}] {w.name}: "
-                        f"1 layer, {w.n_q_heads}q/{w.n_kv_heads}kv heads, D {w.head_dim}, "
+            "workload": f"configs[{3 if (w.name == '128k' and n_layers == 32) else WORKLOAD_INDEX[w.name]}] "
+                        f"{w.name}: {n_layers} layer{'s' if n_layers > 1 else ''}, {w.n_q_heads}q/{w.n_kv_heads}kv heads, D {w.head_dim}, "
                         f"{w.dram_tokens}-token prefix in pinned host DRAM ({w.n_dram_pages} pages/head), "
                         f"local {w.local_cache}, LRU {w.lru_tokens} tokens, top-k {w.top_k_tokens} tokens",
-            "launch": "eager" if args.eager else f"hip-graph replay, {spg} decode steps per graph",
+            "launch": ("eager" if args.eager else
+                       f"hip-graph replay, {spg} decode steps per graph" if n_layers == 1 else
+                       f"hip-graph replay, one model step ({n_layers} layer steps) per graph"),
+            "model_steps_per_s": args.steps / dt,
             "page_stream": "serialised" if args.no_overlap else "in the launch of the first attention pass",
             "seed": args.seed,
         },
@@ -474,7 +494,7 @@ def main():
     if args.cpu_steps > 0:
         result["cpu_baseline"] = cpu_baseline(w, layer, args.cpu_steps)
     if args.reference_shaped_steps > 3 and isinstance(layer.m.lru_cache, LRUCache):
-        del layer
+        del layer, layers, model_step
         torch.cuda.empty_cache()
         ref = reference_shaped(w, args.seed, args.reference_shaped_steps, dev)
         ref["speedup_of_value"] = result["value"] / ref["value"]
