@@ -243,6 +243,47 @@ def cpu_baseline(w, layer, steps):
                       f"{dt / steps * 1e3:.1f} ms/step"}
 
 
+def time_cache_build(layer, dev):
+    """One-time set-up kernels at the size of the workload, timed with events: the page
+    summaries, and the kernel that packs the prompt's K/V into the pinned page store
+    and the initial slots (writes cross the host link once)."""
+    from dram_attention_amd import LRUCache, _lib
+    from dram_attention_amd.topk_selector import page_min_max
+
+    lru, w = layer.m.lru_cache, layer.w
+    if not isinstance(lru, LRUCache) or layer.prompt is None:
+        return None
+    S = w.dram_tokens
+    k = layer.prompt.k[0, :S].to(dev).transpose(0, 1)      # (Hkv, S, D) views, as init_cache passes
+    v = layer.prompt.v[0, :S].to(dev).transpose(0, 1)
+    esz = k.element_size()
+    dram, dram_ptr, hbm = lru.page_stores()
+    scratch_hbm = torch.empty_like(hbm)                    # the live slots must stay as they are
+    lib = _lib.load()
+
+    def build():
+        _lib.check(lib.da_pages_build(
+            k.data_ptr(), v.data_ptr(), k.stride(1), k.stride(0), w.n_kv_heads, w.n_dram_pages,
+            w.page_size, w.head_dim, _lib.dtype_code(w.dtype), dram_ptr, dram.stride(0) * esz,
+            dram.stride(1) * esz, scratch_hbm.data_ptr(), hbm.stride(0) * esz, hbm.stride(1) * esz,
+            w.n_dram_pages - w.n_hbm_pages, w.n_hbm_pages, _lib.stream_ptr(dev)), "da_pages_build")
+
+    res = {}
+    for name, fn in (("page_minmax", lambda: page_min_max(k, w.n_dram_pages)), ("pages_build", build)):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(3):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        res[name + "_ms"] = e0.elapsed_time(e1) / 3
+    res["host_store_bytes"] = dram.numel() * esz
+    res["pages_build_to_host_GBps"] = res["host_store_bytes"] / (res["pages_build_ms"] * 1e-3) / 1e9
+    return res
+
+
 def reference_shaped(w, seed, steps, dev):
     """Stand-in for the reference's own GPU decode step (its Triton and flash-attn
     kernels cannot run here): the same sequence of stages in the same shape,
@@ -491,6 +532,9 @@ def main():
                         "frac_of_link": stream_gbps / link if link else None,
                         "hit_rate": 1.0 - miss_per_step / requests},
     }
+    build = time_cache_build(layer, dev)
+    if build is not None:
+        result["cache_build"] = build
     if args.cpu_steps > 0:
         result["cpu_baseline"] = cpu_baseline(w, layer, args.cpu_steps)
     if args.reference_shaped_steps > 3 and isinstance(layer.m.lru_cache, LRUCache):

@@ -31,6 +31,11 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_int64, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p],
     ),
+    "da_pages_build": (
+        c_int,
+        [c_void_p, c_void_p, c_int64, c_int64, c_int, c_int64, c_int, c_int, c_int, c_void_p,
+         c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],
+    ),
     "da_page_score": (
         c_int,
         [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int64,

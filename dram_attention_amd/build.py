@@ -18,6 +18,7 @@ LIB_PATH = HERE / "libdramattn.so"
 SOURCES = (
     "api.hip",
     "page_minmax.hip",
+    "pages_build.hip",
     "page_score.hip",
     "topk_pages.hip",
     "lru_update.hip",

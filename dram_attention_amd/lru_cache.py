@@ -84,12 +84,6 @@ class LRUCache(torch.nn.Module):
         dram = torch.empty((num_kv_heads, num_dram_pages, page_dim), dtype=dtype, device="cpu",
                            pin_memory=True)
         self.register_buffer("dram_kv_cache", dram)
-        paged = dram.view(num_kv_heads, num_dram_pages, page_size, 2, head_dim)
-        paged[..., 0, :].copy_(k_cache.reshape(num_kv_heads, num_dram_pages, page_size, head_dim),
-                               non_blocking=True)
-        paged[..., 1, :].copy_(v_cache.reshape(num_kv_heads, num_dram_pages, page_size, head_dim),
-                               non_blocking=True)
-
         self.register_buffer(
             "hbm_kv_cache",
             torch.empty(num_kv_heads, num_hbm_pages, page_dim, dtype=dtype, device=device))
@@ -105,15 +99,41 @@ class LRUCache(torch.nn.Module):
         assert num_hbm_pages <= num_dram_pages, "HBM cache size must be smaller than DRAM cache size."
 
         # Start with the most recent pages resident: slot s holds page P - N + s.
-        if k_cache.is_cuda or v_cache.is_cuda:
-            torch.cuda.current_stream(self.hbm_kv_cache.device).synchronize()  # D2H copies above
         first = num_dram_pages - num_hbm_pages
-        self.hbm_kv_cache.copy_(dram[:, first:], non_blocking=True)
+        row_bytes = head_dim * k_cache.element_size()
+        if (k_cache.is_cuda and v_cache.is_cuda and row_bytes % 16 == 0 and num_dram_pages > 0
+                and k_cache.stride(-1) == 1 and v_cache.stride(-1) == 1
+                and k_cache.stride() == v_cache.stride()
+                and all(st * k_cache.element_size() % 16 == 0 for st in k_cache.stride()[:2])
+                and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0):
+            # one kernel packs every page into the pinned store and the resident ones into slots
+            esz = k_cache.element_size()
+            self._dram_device_ptr = _lib.device_visible_ptr(dram)
+            _lib.check(
+                _lib.load().da_pages_build(
+                    k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(1), k_cache.stride(0),
+                    num_kv_heads, num_dram_pages, page_size, head_dim, _lib.dtype_code(dtype),
+                    self._dram_device_ptr, dram.stride(0) * esz, dram.stride(1) * esz,
+                    self.hbm_kv_cache.data_ptr(), self.hbm_kv_cache.stride(0) * esz,
+                    self.hbm_kv_cache.stride(1) * esz, first, num_hbm_pages,
+                    _lib.stream_ptr(self.hbm_kv_cache.device)),
+                "da_pages_build")
+            torch.cuda.current_stream(self.hbm_kv_cache.device).synchronize()  # host store complete
+        else:
+            # host-resident or oddly shaped inputs: torch copies, then the slots from the store
+            self._dram_device_ptr = None
+            paged = dram.view(num_kv_heads, num_dram_pages, page_size, 2, head_dim)
+            paged[..., 0, :].copy_(
+                k_cache.reshape(num_kv_heads, num_dram_pages, page_size, head_dim), non_blocking=True)
+            paged[..., 1, :].copy_(
+                v_cache.reshape(num_kv_heads, num_dram_pages, page_size, head_dim), non_blocking=True)
+            if k_cache.is_cuda or v_cache.is_cuda:
+                torch.cuda.current_stream(self.hbm_kv_cache.device).synchronize()  # D2H copies
+            self.hbm_kv_cache.copy_(dram[:, first:], non_blocking=True)
         slots = torch.arange(num_hbm_pages, dtype=torch.int64, device=device)
         self.dram_page_to_hbm_page_mapping[:, first:] = slots
         self.hbm_page_to_dram_page_mapping[:] = slots + first
 
-        self._dram_device_ptr = None
         self._scratch = None
         self._topk_idx = None
 

@@ -70,6 +70,25 @@ int da_page_minmax(const void *k, int64_t k_head_stride, int64_t k_tok_stride,
                    int dtype, void *out, void *stream);
 
 /*
+ * Subsystem 1b — build the paged KV store from the prompt's keys and values.
+ * Replaces the torch copies of LRUCache.__init__, dram_attention/lru_cache.py:131-141
+ * (interleaved page layout in the pinned store) and :191-209 (initial slots).
+ *   k, v  : (Hkv, n_pages*page_size, D) views, element strides (head_stride,
+ *           tok_stride, 1)
+ *   dram  : device-visible base of the (Hkv, n_pages, page_size*2*D) page store
+ *           (token t of a page: K row at t*2D, V row at t*2D+D), or NULL
+ *   hbm   : base of the slot array, or NULL; page p lands in slot
+ *           p - first_resident_page when that is in [0, n_slots)
+ * Strides of dram / hbm in bytes.  Rows must be a multiple of 16 bytes
+ * (DA_ENOTSUP otherwise).
+ */
+int da_pages_build(const void *k, const void *v, int64_t tok_stride, int64_t head_stride,
+                   int n_kv_heads, int64_t n_pages, int page_size, int head_dim, int dtype,
+                   void *dram, int64_t dram_head_stride_bytes, int64_t dram_page_stride_bytes,
+                   void *hbm, int64_t hbm_head_stride_bytes, int64_t hbm_slot_stride_bytes,
+                   int64_t first_resident_page, int64_t n_slots, void *stream);
+
+/*
  * Subsystem 2 — Quest upper-bound page score
  *     score[n,h,l] = sum_d max(q[n,h,d]*mm[h,l,0,d], q[n,h,d]*mm[h,l,1,d]).
  * Replaces _max_inner_product_kernel / max_inner_product in

@@ -63,6 +63,32 @@ def test_lru_cache_different_page_sizes(page_size):
     assert cache.top_k_selector.chunk_min_max.shape == (4, 1024 * 8 // page_size, 2, 64)
 
 
+@pytest.mark.parametrize("dtype,H,S,D,page,lru", [
+    (torch.bfloat16, 8, 4096, 128, 16, 1024), (torch.float32, 2, 512, 64, 8, 64),
+    (torch.float16, 3, 960, 64, 32, 320), (torch.float32, 2, 256, 24, 16, 64),   # D=24: rows of 96 B
+    (torch.bfloat16, 2, 256, 36, 16, 32),                                       # rows of 72 B: torch copies
+])
+def test_page_store_build_matches_layout(dtype, H, S, D, page, lru):
+    """Pinned page store and initial slots, from the strided views init_cache hands
+    over: token t of page p holds K[h, p*page+t] then V[h, p*page+t]; slot s holds
+    page P - N + s; the maps say so."""
+    from dram_attention_amd import LRUCache
+
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn(S, H, D, generator=g).to(dtype)
+    v = torch.randn(S, H, D, generator=g).to(dtype)
+    cache = LRUCache(k.to(DEV).transpose(0, 1), v.to(DEV).transpose(0, 1), page_size=page,
+                     top_k=4 * page, lru_hbm_cache_size=lru)
+    P, N = S // page, lru // page
+    want = O.pack_pages(k.transpose(0, 1), v.transpose(0, 1), page)
+    assert cache.dram_kv_cache.is_pinned() and same(cache.dram_kv_cache, want)
+    assert same(cache.hbm_kv_cache.cpu(), want[:, P - N:])
+    assert same(cache.hbm_page_to_dram_page_mapping.cpu(),
+                torch.arange(P - N, P).repeat(H, 1))
+    d2h = cache.dram_page_to_hbm_page_mapping.cpu()
+    assert (d2h[:, :P - N] == -1).all() and same(d2h[:, P - N:], torch.arange(N).repeat(H, 1))
+
+
 def test_lru_cache_invalid_initialization_and_hbm_size():
     from dram_attention_amd import LRUCache
 
