@@ -248,6 +248,15 @@ class DRAMAttention(torch.nn.Module):
             self.lru_cache = DummyCache(k_cache=prefix_k, v_cache=prefix_v, device=self.device)
         self._workspace = None
 
+    def init_cache_from_file(self, cache_dir: str, index: int) -> int:
+        """init_cache from the chat example's per-layer file ``NN_cache.pth``; returns
+        the prompt length (the position of the first generated token)."""
+        from .kv_file import load_layer_cache
+
+        k, v = load_layer_cache(cache_dir, index, self.device)
+        self.init_cache(k.to(self.cache_k.dtype), v.to(self.cache_v.dtype))
+        return k.shape[1]
+
     def forward(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, *, start_pos,
                 stage: str):
         bsz, seqlen, H, D = xq.shape

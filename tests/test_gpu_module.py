@@ -138,6 +138,33 @@ def test_module_init_and_errors():
         m(x2, x2, x2, start_pos=0, stage="prefill")
 
 
+def test_init_cache_from_layer_file(tmp_path):
+    """A layer set up from the chat example's cache file decodes like one set up from
+    the tensors themselves."""
+    from dram_attention_amd import DRAMAttention, save_layer_cache
+
+    w = WORKLOADS["128k"].scaled(dram_tokens=4096, local_cache=256, lru_tokens=1024,
+                                 top_k_tokens=256, steps=3)
+    prompt = make_prompt(w, 11)
+    save_layer_cache(str(tmp_path), 3, prompt.k, prompt.v)
+    mods = []
+    for from_file in (True, False):
+        m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                          w.n_kv_heads, w.head_dim, device=DEV, dtype=w.dtype)
+        if from_file:
+            assert m.init_cache_from_file(str(tmp_path), 3) == w.prompt_tokens
+        else:
+            m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+        mods.append(m)
+    assert same(mods[0].lru_cache.dram_kv_cache, mods[1].lru_cache.dram_kv_cache)
+    inputs = DecodeInputs(w, prompt.q0, 11)
+    for t in range(w.steps):
+        xq, xk, xv = (x.to(DEV) for x in inputs.next())
+        a = mods[0](xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
+        b = mods[1](xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
+        assert same(a, b)
+
+
 def test_module_prefill_then_generate_shapes():
     """The reference's prefill/generate smoke at its 66K-token shape."""
     m = make_module()

@@ -129,3 +129,26 @@ def test_synthetic_workloads():
     for _ in range(3):
         for x, y in zip(a.next(), b.next()):
             assert torch.equal(x, y)
+
+
+def test_layer_cache_file_round_trip(tmp_path):
+    """The chat example's per-layer file: name, keys, shapes and dtype survive a
+    write / memory-mapped read, and malformed files are refused."""
+    import torch
+
+    from dram_attention_amd import layer_cache_path, load_layer_cache, save_layer_cache
+
+    g = torch.Generator().manual_seed(0)
+    k = torch.randn(1, 100, 2, 16, generator=g).bfloat16()
+    v = torch.randn(1, 100, 2, 16, generator=g).bfloat16()
+    path = save_layer_cache(str(tmp_path), 7, k, v)
+    assert path == layer_cache_path(str(tmp_path), 7) and path.endswith("07_cache.pth")
+    raw = torch.load(path, weights_only=True)
+    assert set(raw) == {"cache_k", "cache_v"} and raw["cache_k"].device.type == "cpu"
+    k2, v2 = load_layer_cache(str(tmp_path), 7, device="cpu")
+    assert k2.dtype == torch.bfloat16 and torch.equal(k2, k) and torch.equal(v2, v)
+    with pytest.raises(ValueError):
+        save_layer_cache(str(tmp_path), 8, k[0], v[0])
+    torch.save({"cache_k": k}, layer_cache_path(str(tmp_path), 9))
+    with pytest.raises(KeyError):
+        load_layer_cache(str(tmp_path), 9, device="cpu")
