@@ -121,12 +121,45 @@ def run_topk(scores, rep, k):
 @pytest.mark.parametrize("rows,rep,H,L,k", [(4, 4, 8, 8192, 256), (2, 2, 2, 512, 32),
                                             (3, 1, 2, 1000, 1000), (6, 3, 1, 77, 5),
                                             (1, 1, 1, 1, 1), (2, 1, 2, 5000, 1),
-                                            (8, 8, 2, 20000, 512), (1, 1, 1, 300, 299)])
+                                            (8, 8, 2, 20000, 512), (1, 1, 1, 300, 299),
+                                            (2, 1, 1, 65536, 8192), (8, 8, 1, 65536, 512),
+                                            (1, 1, 1, 16385, 600)])
 def test_topk_pages_exact(rows, rep, H, L, k):
     scores = torch.randn(rows, H, L, generator=gen(13))
     got = run_topk(scores, rep, k)
     want = O.select_pages(scores, rows // rep, rep, k)
     assert same(got, want)
+
+
+def test_topk_pages_bf16_rounded_scores_at_1m_row_length():
+    """65 536 pages per row with scores that share their low 16 bits (rounded to
+    bf16, as the selector produces them): many exact ties, lowest index first."""
+    scores = (torch.randn(4, 2, 65536, generator=gen(15)) * 8).bfloat16().float()
+    got = run_topk(scores, 4, 512)
+    want = torch.sort(scores, dim=-1, descending=True, stable=True).indices[..., :512]
+    assert same(got[0], want.transpose(0, 1))
+
+
+def test_empty_inputs_are_no_ops():
+    """Zero rows, zero pages, zero requests: every entry point returns without a launch."""
+    from dram_attention_amd import max_inner_product
+    from dram_attention_amd.lru_kernel import LruScratch, lru_update_and_gather
+
+    assert max_inner_product(torch.zeros(0, 2, 64, device=DEV), torch.zeros(2, 8, 2, 64, device=DEV)).shape == (0, 2, 8)
+    assert max_inner_product(torch.zeros(3, 2, 64, device=DEV), torch.zeros(2, 0, 2, 64, device=DEV)).shape == (3, 2, 0)
+    H, P, N = 2, 8, 4
+    dram = torch.randn(H, P, 32, device=DEV)
+    hbm = dram[:, P - N:].clone()
+    time = torch.zeros(H, N, device=DEV)
+    d2h = torch.full((H, P), -1, dtype=torch.int64, device=DEV)
+    d2h[:, P - N:] = torch.arange(N, device=DEV)
+    h2d = torch.arange(P - N, P, device=DEV).repeat(H, 1)
+    step = torch.zeros(1, dtype=torch.int32, device=DEV)
+    before = (hbm.clone(), d2h.clone(), h2d.clone())
+    lru_update_and_gather(dram, time, d2h, h2d, torch.zeros(H, 0, dtype=torch.int64, device=DEV), step,
+                          hbm, LruScratch.allocate(H, 0, DEV), bump_step=True)
+    torch.cuda.synchronize()
+    assert step.item() == 1 and same(hbm, before[0]) and same(d2h, before[1]) and same(h2d, before[2])
 
 
 @pytest.mark.parametrize("levels", [2, 7, 200])
