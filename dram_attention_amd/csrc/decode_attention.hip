@@ -434,7 +434,7 @@ struct GatherAttendArgs {
   int K;
   const char *q;
   int64_t q_head_stride;
-  int rep, n_q_heads;
+  int rep, n_q_heads, n_kv_heads;
   float scale_log2;
   float *part_ml, *part_acc;
   int chunk0;
@@ -443,6 +443,22 @@ struct GatherAttendArgs {
 constexpr int kGatherThreads = 256;
 constexpr int kGatherMaxLoads = 4;  // 16-byte loads per lane and page: pages up to 16 KiB
 constexpr int kGatherIdBatch = 1024;  // miss-list entries of a block staged in LDS at a time
+
+// The page stream's blocks share the miss lists of all kv heads, taken as one
+// list in head order, in equal contiguous ranges (heads miss unequally: the
+// busiest head of a step has ~20 % more pages than the average, and a stream
+// split per head would end with a few blocks and an idle host link).  With
+// `total` entries and `n_blocks` blocks, n_eff = min(n_blocks, total) of them
+// work, block b on entries [b*total/n_eff, (b+1)*total/n_eff).  A block that
+// crosses a head boundary leaves one partial per head it touched.
+struct StreamRange {
+  int64_t begin, end;
+};
+__device__ __forceinline__ StreamRange stream_range(int b, int n_blocks, int64_t total) {
+  const int64_t n_eff = total < n_blocks ? total : n_blocks;
+  if (b >= n_eff) return {0, 0};
+  return {b * total / n_eff, (b + 1) * total / n_eff};
+}
 
 template <typename T, int kLanes, int kRows>
 __device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, const int block_x,
@@ -457,9 +473,24 @@ __device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, c
   const int within = tid % kTokLanes;
   const bool is_v = within >= kLanes;
   const int c = within % kLanes;
-  const int h = blockIdx.y;
+  // this block's range of the concatenated miss lists
+  int64_t total = 0;
+  for (int hh = 0; hh < g.n_kv_heads; ++hh) total += g.miss_count[hh];
+  const StreamRange range = stream_range(block_x, n_blocks, total);
+  if (range.begin >= range.end) return;  // the merge does not count this block either
+
+  __shared__ int32_t sm_slot[kGatherIdBatch], sm_page[kGatherIdBatch];
+  __shared__ float sm_m[kWaves][kRows];
+  __shared__ float sm_l[kWaves][kRows];
+  __shared__ float sm_acc[kWaves][kRows][D];
+  int64_t head_off = 0;
+  for (int h = 0; h < g.n_kv_heads; ++h) {
   const int n_miss = g.miss_count[h];
-  if (block_x >= n_miss) return;  // the merge does not count this block either
+  const int64_t lo64 = (range.begin > head_off ? range.begin : head_off) - head_off;
+  const int64_t hi64 = (range.end < head_off + n_miss ? range.end : head_off + n_miss) - head_off;
+  head_off += n_miss;
+  if (lo64 >= hi64) continue;  // uniform: nothing of this head in the range
+  const int first = (int)lo64, n_mine = (int)(hi64 - lo64);
 
   u32x4 qv[kRows];
 #pragma unroll
@@ -481,8 +512,6 @@ __device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, c
   // This block's entries (slot, page), staged in LDS a batch at a time: a page's
   // loads then depend on no other global load, and the next page is always in
   // flight while the current one is stored and attended.
-  __shared__ int32_t sm_slot[kGatherIdBatch], sm_page[kGatherIdBatch];
-  const int n_mine = (n_miss - block_x + n_blocks - 1) / n_blocks;
   // Issues the loads of this block's n-th staged entry; dst == nullptr marks a
   // superseded one.  Always kGatherMaxLoads loads per lane, lanes with nothing to
   // fetch reading the query instead: with a fixed count the wait for one page's
@@ -534,7 +563,7 @@ __device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, c
     const int n_batch = n_mine - batch0 < kGatherIdBatch ? n_mine - batch0 : kGatherIdBatch;
     __syncthreads();  // the previous batch is no longer read
     for (int n = tid; n < n_batch; n += kGatherThreads) {
-      const int64_t i = (int64_t)block_x + (int64_t)(batch0 + n) * n_blocks;
+      const int64_t i = (int64_t)first + batch0 + n;
       sm_slot[n] = mslot[i];
       sm_page[n] = mpage[i];
     }
@@ -570,9 +599,6 @@ __device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, c
     }
   }
   // Merge the waves through LDS; the value lanes of a wave's first token hold its state.
-  __shared__ float sm_m[kWaves][kRows];
-  __shared__ float sm_l[kWaves][kRows];
-  __shared__ float sm_acc[kWaves][kRows][D];
   if (is_v && lane < kTokLanes) {
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
@@ -606,12 +632,14 @@ __device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, c
       g.part_ml[slot * 2 + 1] = lt;
     }
   }
+  }  // heads in this block's range (the next head's first barrier retires these reads)
 }
 
 template <typename T, int kLanes, int kRows>
 __global__ void __launch_bounds__(kGatherThreads)
 pages_gather_attend_kernel(const GatherAttendArgs g) {
-  gather_attend_block<T, kLanes, kRows>(g, blockIdx.x, gridDim.x);
+  gather_attend_block<T, kLanes, kRows>(g, blockIdx.y * gridDim.x + blockIdx.x,
+                                        gridDim.x * gridDim.y);
 }
 
 // Both of the above in one launch: blocks [0, g_blocks) of every kv head run the
@@ -624,7 +652,9 @@ template <typename T, int kLanes, int kRowsAttn, int kRowsGather>
 __global__ void __launch_bounds__(kAttnThreads)
 decode_stream_attend_kernel(const AttnArgs a, const GatherAttendArgs g, const int g_blocks) {
   if ((int)blockIdx.x < g_blocks) {
-    if (blockIdx.z == 0) gather_attend_block<T, kLanes, kRowsGather>(g, blockIdx.x, g_blocks);
+    if (blockIdx.z == 0)
+      gather_attend_block<T, kLanes, kRowsGather>(g, blockIdx.y * g_blocks + blockIdx.x,
+                                                  g_blocks * gridDim.y);
   } else {
     attention_split_block<T, kLanes, kRowsAttn, false>(a, (int)blockIdx.x - g_blocks);
   }
@@ -657,10 +687,31 @@ decode_attention_merge_kernel(const AttnArgs a, int mode, int head_dim, char *__
   int n_t = 0;                                              // live tail chunks
   int tail_chunk0 = a.n_pchunks + a.n_lchunks;
   if (a.gather_blocks > 0 && mode != kMergePre) {
-    // block b of the gather pass wrote a partial iff it had an entry to copy
-    const int misses = a.miss_count[hq / a.rep];
-    n_t = misses < a.gather_blocks ? misses : a.gather_blocks;
-    tail_chunk0 = a.gather_chunk0;
+    // the blocks of the page stream whose range met this kv head's miss list
+    const int n_kv = a.n_q_heads / a.rep, hk = hq / a.rep;
+    const int n_blocks = a.gather_blocks * n_kv;
+    int64_t total = 0, off = 0;
+    for (int hh = 0; hh < n_kv; ++hh) {
+      const int mc = a.miss_count[hh];
+      if (hh < hk) off += mc;
+      total += mc;
+    }
+    const int64_t mine = a.miss_count[hk];
+    if (mine > 0) {
+      // entry x lies in block ceil((x+1)*n_eff/total) - 1 (ranges are floor(b*total/n_eff))
+      const int64_t n_eff = total < n_blocks ? total : n_blocks;
+      int64_t b_first, b_last;
+      if (total < (1 << 24)) {  // the usual case: 32-bit divisions (n_eff <= 64)
+        const uint32_t t32 = (uint32_t)total, n32 = (uint32_t)n_eff;
+        b_first = (((uint32_t)off + 1u) * n32 + t32 - 1u) / t32 - 1u;
+        b_last = ((uint32_t)(off + mine) * n32 + t32 - 1u) / t32 - 1u;
+      } else {
+        b_first = ((off + 1) * n_eff + total - 1) / total - 1;
+        b_last = ((off + mine) * n_eff + total - 1) / total - 1;
+      }
+      n_t = (int)(b_last - b_first + 1);
+      tail_chunk0 = a.gather_chunk0 + (int)b_first;
+    }
   } else if (a.n_tchunks > 0 && mode != kMergePre) {
     const int64_t tail = (int64_t)a.miss_count[hq / a.rep] * a.page_size;
     n_t = (int)((tail + a.tail_chunk - 1) / a.tail_chunk);
@@ -767,7 +818,7 @@ static int lanes_of(int head_dim, int dtype) {
   return (lanes >= 4 && lanes <= 64 && is_pow2(lanes)) ? lanes : 0;
 }
 
-constexpr int kGatherMaxBlocks = 64;  // per kv head
+constexpr int kGatherMaxBlocks = 64;  // blocks of a page stream, all kv heads together
 
 struct ChunkPlan {
   int chunk, tail_chunk, n_p, n_l, n_t;
@@ -944,9 +995,9 @@ extern "C" int da_pages_gather_attend(
              "da_pages_gather_attend: unknown dtype %d", dtype);
   DA_REQUIRE(dram && hbm && miss_page && miss_slot && miss_count && q && workspace,
              "da_pages_gather_attend: null pointer");
-  DA_REQUIRE(blocks_per_head >= 1 && blocks_per_head <= kGatherMaxBlocks,
-             "da_pages_gather_attend: blocks_per_head %d not in 1..%d", blocks_per_head,
-             kGatherMaxBlocks);
+  DA_REQUIRE(blocks_per_head >= 1 && (int64_t)blocks_per_head * n_kv_heads <= kGatherMaxBlocks,
+             "da_pages_gather_attend: blocks_per_head %d x %d kv heads not in 1..%d",
+             blocks_per_head, n_kv_heads, kGatherMaxBlocks);
   const int lanes = lanes_of(head_dim, dtype);
   const int rep = n_q_heads / n_kv_heads;
   const int64_t page_vecs = (int64_t)page_size * 2 * lanes;
@@ -982,6 +1033,7 @@ extern "C" int da_pages_gather_attend(
   g.q_head_stride = q_head_stride;
   g.rep = rep;
   g.n_q_heads = n_q_heads;
+  g.n_kv_heads = n_kv_heads;
   g.scale_log2 = scale * kLog2e;
   g.part_acc = (float *)workspace;
   g.part_ml = g.part_acc + (size_t)p.total() * n_q_heads * head_dim;
@@ -1094,10 +1146,11 @@ extern "C" int da_decode_attention_paged(
     a.miss_capacity = overlap->miss_capacity;
     miss_tokens = (int64_t)overlap->miss_capacity * overlap->page_size;
     phase = overlap->phase;
-    DA_REQUIRE(overlap->gather_blocks >= 0 && overlap->gather_blocks <= kGatherMaxBlocks &&
+    DA_REQUIRE(overlap->gather_blocks >= 0 &&
+                   (int64_t)overlap->gather_blocks * n_kv_heads <= kGatherMaxBlocks &&
                    (overlap->gather_blocks == 0 || miss_tokens > 0),
-               "da_decode_attention: gather_blocks %d out of range (at most %d)",
-               overlap->gather_blocks, kGatherMaxBlocks);
+               "da_decode_attention: gather_blocks %d x %d kv heads out of range (at most %d)",
+               overlap->gather_blocks, n_kv_heads, kGatherMaxBlocks);
     a.gather_blocks = overlap->gather_blocks;
   }
   const ChunkPlan p = plan_chunks(n_kv_heads, lanes, p_len, c_capacity, miss_tokens);
@@ -1148,6 +1201,7 @@ extern "C" int da_decode_attention_paged(
     g.q_head_stride = q_head_stride;
     g.rep = a.rep;
     g.n_q_heads = n_q_heads;
+    g.n_kv_heads = n_kv_heads;
     g.scale_log2 = a.scale_log2;
     g.part_acc = a.part_acc;
     g.part_ml = a.part_ml;

@@ -129,7 +129,7 @@ def gather_attend_supported(n_q_heads: int, n_kv_heads: int, head_dim: int, page
     """Whether pages_gather_attend takes this shape (else: pages_gather + tail pass)."""
     row = head_dim * torch.empty(0, dtype=dtype).element_size()
     return (row in (64, 128, 256, 512) and n_q_heads // n_kv_heads <= 8
-            and page_size * 2 * row <= 16384)
+            and page_size * 2 * row <= 16384 and n_kv_heads <= 64)
 
 
 def pages_gather_attend(dram_kv_cache: torch.Tensor, hbm_kv_cache: torch.Tensor,

@@ -306,11 +306,13 @@ int da_decode_attention_paged(const void *q, int64_t q_head_stride, int n_q_head
  *   workspace   : the workspace of this step's da_decode_attention_paged calls
  *                 (same p_len, c_capacity, and miss_capacity = k); every block
  *                 with an entry to copy leaves one partial result in it
- *   blocks_per_head : workgroups per kv head, 1..64 (few fat ones: 32 in all
- *                 saturate the host link); pass the same value as
+ *   blocks_per_head : workgroups per kv head; blocks_per_head * Hkv <= 64 (few
+ *                 fat ones: 32 in all saturate the host link).  The blocks
+ *                 share the miss lists of all heads in equal parts, whatever
+ *                 each head's count.  Pass the same value as
  *                 da_paged_overlap.gather_blocks to DA_PHASE_SECOND
  * DA_ENOTSUP when rows are not 64..512 bytes, Hq / Hkv > 8 or a page exceeds
- * 16 KiB: use da_pages_gather and the tail pass of DA_PHASE_SECOND then.
+ * 16 KiB (and Hkv > 64 leaves no valid blocks_per_head): use da_pages_gather and the tail pass of DA_PHASE_SECOND then.
  */
 int da_pages_gather_attend(const void *dram, int64_t dram_head_stride_bytes,
                            int64_t dram_page_stride_bytes, void *hbm,
