@@ -284,6 +284,14 @@ def test_decode_parity_wide_gqa_group_takes_the_tail_pass():
     run_parity(w, 5, w.steps, atol=2e-2, rtol=1e-2)
 
 
+def test_decode_parity_page_size_not_a_power_of_two():
+    """24-token pages: no shift for the page index, three 16-byte loads per lane and
+    page in the stream, chunks that straddle pages in the first pass."""
+    w = WORKLOADS["128k"].scaled(dram_tokens=24 * 320, local_cache=24 * 20, lru_tokens=24 * 96,
+                                 top_k_tokens=24 * 12, steps=5, page_size=24)
+    run_parity(w, 9, w.steps, atol=2e-2, rtol=1e-2)
+
+
 def test_page_stream_overlap_changes_nothing():
     """Attention issued around a concurrent page stream (two phases, side stream)
     gives the bits of the serialised order, and both agree with one plain pass."""
