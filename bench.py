@@ -532,17 +532,29 @@ def main():
                         "frac_of_link": stream_gbps / link if link else None,
                         "hit_rate": 1.0 - miss_per_step / requests},
     }
-    build = time_cache_build(layer, dev)
-    if build is not None:
-        result["cache_build"] = build
+    # The auxiliary legs below must never cost the headline line: a failure in one of
+    # them is reported in its place.
+    def leg(name, fn):
+        try:
+            value = fn()
+            if value is not None:
+                result[name] = value
+        except Exception as exc:  # noqa: BLE001 - reported, not swallowed
+            result[name] = {"error": f"{type(exc).__name__}: {exc}"}
+
+    leg("cache_build", lambda: time_cache_build(layer, dev))
     if args.cpu_steps > 0:
-        result["cpu_baseline"] = cpu_baseline(w, layer, args.cpu_steps)
+        leg("cpu_baseline", lambda: cpu_baseline(w, layer, args.cpu_steps))
     if args.reference_shaped_steps > 3 and isinstance(layer.m.lru_cache, LRUCache):
         del layer, layers, model_step
         torch.cuda.empty_cache()
-        ref = reference_shaped(w, args.seed, args.reference_shaped_steps, dev)
-        ref["speedup_of_value"] = result["value"] / ref["value"]
-        result["reference_shaped_gpu"] = ref
+
+        def ref_leg():
+            ref = reference_shaped(w, args.seed, args.reference_shaped_steps, dev)
+            ref["speedup_of_value"] = result["value"] / ref["value"]
+            return ref
+
+        leg("reference_shaped_gpu", ref_leg)
     print(json.dumps(result))
     return 0
 
