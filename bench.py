@@ -233,12 +233,13 @@ def cpu_baseline(w, layer, steps):
                        w.n_kv_heads, w.head_dim, dtype=w.dtype)
     o.init_cache(layer.prompt.k, layer.prompt.v)
     qs, ks, vs = layer.host_inputs
+    stages = {}
     t0 = time.perf_counter()
     for t in range(steps):
-        o.generate(qs[t], ks[t], vs[t], w.prompt_tokens + t)
+        o.generate(qs[t], ks[t], vs[t], w.prompt_tokens + t, timings=stages)
     dt = time.perf_counter() - t0
     return {"value": steps / dt, "unit": "decode steps/s per layer", "cores": torch.get_num_threads(),
-            "kind": "port",
+            "kind": "port", "stage_ms_per_step": {k: v / steps * 1e3 for k, v in stages.items()},
             "sample": f"first {steps} decode steps of workload {w.name}, torch-CPU oracle, "
                       f"{dt / steps * 1e3:.1f} ms/step"}
 

@@ -33,6 +33,7 @@ stated "given identical scores".
 from __future__ import annotations
 
 import math
+import time
 from dataclasses import dataclass
 from typing import Optional, Tuple
 
@@ -298,22 +299,31 @@ class DecodeOracle:
         else:
             self.static_k, self.static_v = pk, pv
 
-    def select(self, xq: torch.Tensor, scores: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def select(self, xq: torch.Tensor, scores: Optional[torch.Tensor] = None,
+               timings: Optional[dict] = None) -> torch.Tensor:
         """(Hkv, rep*kp) page list of this step; `scores` overrides the oracle's own
         (seq*rep, Hkv, P) scores (used to test selection on identical scores)."""
         bsz, seq, Hq, D = xq.shape
         rep = Hq // self.n_kv_heads
+        t0 = time.perf_counter()
         if scores is None:
             scores = scores_for_selection(xq, self.min_max)
-        return lru_index_list(select_pages(scores, seq, rep, min(self.kp, self.min_max.shape[1])))
+        t1 = time.perf_counter()
+        idx = lru_index_list(select_pages(scores, seq, rep, min(self.kp, self.min_max.shape[1])))
+        if timings is not None:
+            timings["score"] = timings.get("score", 0.0) + t1 - t0
+            timings["top_k"] = timings.get("top_k", 0.0) + time.perf_counter() - t1
+        return idx
 
     def generate(self, xq, xk, xv, start_pos: int, scores: Optional[torch.Tensor] = None,
-                 idx: Optional[torch.Tensor] = None):
-        """xq (1,1,Hq,D), xk/xv (1,1,Hkv,D) -> (1,1,Hq,D) in xq.dtype."""
+                 idx: Optional[torch.Tensor] = None, timings: Optional[dict] = None):
+        """xq (1,1,Hq,D), xk/xv (1,1,Hkv,D) -> (1,1,Hq,D) in xq.dtype.  `timings`, when
+        given, accumulates seconds per stage (score, top_k, lru, attention)."""
         if self.uses_lru:
             if idx is None:
-                idx = self.select(xq, scores)
+                idx = self.select(xq, scores, timings)
             self.last_idx = idx
+            t0 = time.perf_counter()
             hbm_np = self.hbm.view(torch.int16).numpy() if self.hbm.element_size() == 2 \
                 else self.hbm.numpy()
             dram_np = self.dram.view(torch.int16).numpy() if self.dram.element_size() == 2 \
@@ -321,8 +331,11 @@ class DecodeOracle:
             self.last_hit, self.last_misses = lru_load(
                 self.state, idx.numpy(), self.state.step + 1, dram_np, hbm_np)
             pk, pv = split_hbm_pages(self.hbm, self.page_size, self.head_dim)
+            if timings is not None:
+                timings["lru"] = timings.get("lru", 0.0) + time.perf_counter() - t0
         else:
             pk, pv = self.static_k, self.static_v
+        t0 = time.perf_counter()
         c = int(start_pos) - self.dram_kv_cache_size
         self.cache_k[c] = xk[0, 0]
         self.cache_v[c] = xv[0, 0]
@@ -332,4 +345,7 @@ class DecodeOracle:
                                          self.cache_v[: c + 1].transpose(0, 1))
         if self.round_partials:
             out_p, out_s = out_p.to(self.dtype), out_s.to(self.dtype)
-        return combine(out_p, lse_p, out_s, lse_s, xq.dtype).reshape(1, 1, *q.shape)
+        out = combine(out_p, lse_p, out_s, lse_s, xq.dtype).reshape(1, 1, *q.shape)
+        if timings is not None:
+            timings["attention"] = timings.get("attention", 0.0) + time.perf_counter() - t0
+        return out
