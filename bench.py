@@ -233,13 +233,20 @@ def cpu_baseline(w, layer, steps):
                        w.n_kv_heads, w.head_dim, dtype=w.dtype)
     o.init_cache(layer.prompt.k, layer.prompt.v)
     qs, ks, vs = layer.host_inputs
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            cpu_model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")),
+                             cpu_model)
+    except OSError:
+        pass
     stages = {}
     t0 = time.perf_counter()
     for t in range(steps):
         o.generate(qs[t], ks[t], vs[t], w.prompt_tokens + t, timings=stages)
     dt = time.perf_counter() - t0
     return {"value": steps / dt, "unit": "decode steps/s per layer", "cores": torch.get_num_threads(),
-            "kind": "port", "stage_ms_per_step": {k: v / steps * 1e3 for k, v in stages.items()},
+            "kind": "port", "cpu_model": cpu_model, "stage_ms_per_step": {k: v / steps * 1e3 for k, v in stages.items()},
             "sample": f"first {steps} decode steps of workload {w.name}, torch-CPU oracle, "
                       f"{dt / steps * 1e3:.1f} ms/step"}
 
