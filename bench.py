@@ -9,7 +9,8 @@ attention over the resident pages + local window + new token.  Inputs of all
 steps are staged in HBM before the clock starts.  By default the step is
 captured once into a HIP graph (position and LRU step live on the device) and
 replayed (--steps-per-graph consecutive steps per graph, as a model step of
-several layers would be); --eager issues the launches from Python every step;
+several layers would be, with one input fetch and one counter increment per
+graph); --eager issues the launches from Python every step;
 --no-overlap runs the page stream to completion before attention starts.
 
 Prints ONE JSON line: the BASELINE metric plus `roofline` (the dominant HBM
@@ -88,21 +89,38 @@ class Layer:
         Hq, Hkv, D = w.n_q_heads, w.n_kv_heads, w.head_dim
         self.qkv = torch.cat([self.qs.view(total_steps, Hq * D), self.ks.view(total_steps, Hkv * D),
                               self.vs.view(total_steps, Hkv * D)], dim=1).contiguous()
-        # [step index, position]: both advance with a single increment kernel
-        self.ctr = torch.tensor([0, w.prompt_tokens], dtype=torch.int32, device=dev)
-        self.t_dev, self.pos_dev = self.ctr[0:1], self.ctr[1:2]
+        # Row 0: step index, row 1: position, each for this step and the next few
+        # (column j = j steps ahead); all advance with a single increment kernel.
+        ahead = torch.arange(self.MAX_STEPS_PER_GRAPH, dtype=torch.int32)
+        self.cnt = torch.stack([ahead, ahead + w.prompt_tokens]).to(dev)
+        self.t_dev, self.pos_dev = self.cnt[0, 0:1], self.cnt[1, 0:1]
         self.out = None
 
-    def step_from_device_state(self):
-        """One decode step driven entirely by device-resident counters."""
-        w, m = self.w, self.m
+    MAX_STEPS_PER_GRAPH = 32
+
+    def _step(self, row, pos):
+        w = self.w
         Hq, Hkv, D = w.n_q_heads, w.n_kv_heads, w.head_dim
-        row = self.qkv.index_select(0, self.t_dev)[0]
         xq = row[: Hq * D].view(1, 1, Hq, D)
         xk = row[Hq * D:(Hq + Hkv) * D].view(1, 1, Hkv, D)
         xv = row[(Hq + Hkv) * D:].view(1, 1, Hkv, D)
-        self.out = m(xq, xk, xv, start_pos=self.pos_dev, stage="generate")
-        self.ctr += 1
+        self.out = self.m(xq, xk, xv, start_pos=pos, stage="generate")
+        return self.out
+
+    def step_from_device_state(self):
+        """One decode step driven entirely by device-resident counters."""
+        self._step(self.qkv.index_select(0, self.t_dev)[0], self.pos_dev)
+        self.cnt += 1
+        return self.out
+
+    def steps_from_device_state(self, n):
+        """n consecutive decode steps: their inputs arrive by one fetch and the
+        counters advance once, the way a serving loop hands a model step its
+        inputs and bumps the position once per token, not once per layer."""
+        rows = self.qkv.index_select(0, self.cnt[0, :n])
+        for j in range(n):
+            self._step(rows[j], self.cnt[1, j:j + 1])
+        self.cnt += n
         return self.out
 
 
@@ -146,7 +164,7 @@ def time_kernels(layer, steps):
             torch.cuda.synchronize()
             acc["decode_attention_split"] += e0.elapsed_time(e1)   # includes its merge launch
             local_rows.append(c_len)
-            layer.ctr += 1
+            layer.cnt += 1
         return ({"decode_attention_split": acc["decode_attention_split"] / steps * 1e3}, 0.0,
                 sum(local_rows) / len(local_rows))
 
@@ -204,7 +222,7 @@ def time_kernels(layer, steps):
             acc[name] += e0.elapsed_time(e1) / repeat
         misses += int(lru.last_miss_counts().sum().item())
         local_rows.append(c_len)
-        layer.ctr += 1
+        layer.cnt += 1
     us = {n: v / steps * 1e3 for n, v in acc.items() if v > 0.0}  # microseconds
     if "split+merge" in us:
         us["decode_attention_merge"] = us.pop("split+merge") - us["decode_attention_split"]
@@ -453,12 +471,12 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             model_step()
-        spg = max(1, min(args.steps_per_graph, args.steps)) if n_layers == 1 else 1
+        spg = (max(1, min(args.steps_per_graph, args.steps, Layer.MAX_STEPS_PER_GRAPH))
+               if n_layers == 1 else 1)
         if spg > 1:
             graph_many = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph_many):
-                for _ in range(spg):
-                    model_step()
+                layer.steps_from_device_state(spg)
         # the captures themselves executed nothing; replay for the remaining warm-up steps
         for _ in range(max(args.warmup - 2, 0)):
             graph.replay()
@@ -520,7 +538,8 @@ def main():
                         f"{w.dram_tokens}-token prefix in pinned host DRAM ({w.n_dram_pages} pages/head), "
                         f"local {w.local_cache}, LRU {w.lru_tokens} tokens, top-k {w.top_k_tokens} tokens",
             "launch": ("eager" if args.eager else
-                       f"hip-graph replay, {spg} decode steps per graph" if n_layers == 1 else
+                       f"hip-graph replay, {spg} decode steps per graph (one input fetch and one counter "
+                       f"increment per graph)" if n_layers == 1 else
                        f"hip-graph replay, one model step ({n_layers} layer steps) per graph"),
             "model_steps_per_s": args.steps / dt,
             "page_stream": "serialised" if args.no_overlap else "in the launch of the first attention pass",
