@@ -292,6 +292,21 @@ def test_decode_parity_page_size_not_a_power_of_two():
     run_parity(w, 9, w.steps, atol=2e-2, rtol=1e-2)
 
 
+def test_decode_parity_fp16():
+    w = WORKLOADS["128k"].scaled(dram_tokens=8192, local_cache=512, lru_tokens=2048,
+                                 top_k_tokens=512, steps=6, dtype=torch.float16)
+    run_parity(w, 12, w.steps, atol=4e-3, rtol=1e-2)
+
+
+def test_decode_parity_long_run_with_heavy_eviction():
+    """150 steps on a small cache that turns over many times: every slot is
+    re-assigned repeatedly and the step counter leaves the single digits."""
+    w = WORKLOADS["128k"].scaled(n_q_heads=8, n_kv_heads=2, dram_tokens=4096, local_cache=128,
+                                 lru_tokens=512, top_k_tokens=128, steps=150)
+    rate = run_parity(w, 13, w.steps, atol=2e-2, rtol=1e-2)
+    assert rate < 0.95      # the run really paged
+
+
 def test_page_stream_overlap_changes_nothing():
     """Attention issued around a concurrent page stream (two phases, side stream)
     gives the bits of the serialised order, and both agree with one plain pass."""
