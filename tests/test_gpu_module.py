@@ -349,6 +349,9 @@ def test_page_stream_overlap_changes_nothing():
                   page_size=32, dtype=torch.float16)),
     ("128k", dict(dram_tokens=4096, local_cache=256, lru_tokens=1024, top_k_tokens=128, steps=4,
                   page_size=8, head_dim=64, n_q_heads=4, n_kv_heads=2)),
+    ("cpu", dict(steps=3, head_dim=128)),                       # fp32 rows of 512 bytes: one token per wave
+    ("128k", dict(dram_tokens=4096, local_cache=256, lru_tokens=1024, top_k_tokens=256, steps=3,
+                  n_q_heads=48, n_kv_heads=48, head_dim=64)),   # more kv heads than stream blocks
 ])
 def test_attention_on_the_page_stream_equals_tail_pass(base, kw):
     """Attending over the streamed pages inside the page stream, or in a pass
