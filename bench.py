@@ -13,7 +13,7 @@ several layers would be, with one input fetch and one counter increment per
 graph); --eager issues the launches from Python every step;
 --no-overlap runs the page stream to completion before attention starts.
 
-Prints ONE JSON line: the BASELINE metric plus `roofline` (the dominant HBM
+Prints ONE JSON line: the headline metric plus `roofline` (the dominant HBM
 kernel, timed live with events on the launch stream) and `cpu_baseline` (the CPU
 oracle timed on this box's host cores on a bounded sample of the same workload).
 """
