@@ -213,10 +213,11 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
     DA_LRU_STAMP(4);
   }
 
-  // The last head to finish publishes the bumped step (every head has read the
-  // old value by then) and re-arms the ticket for the next call.
+  // The last head to finish publishes the bumped step and re-arms the ticket for
+  // the next call.  Every head has read the old value by then: its own ticket
+  // comes after that read in program order and depends on nothing another block
+  // wrote, so no fence is needed (the kernel boundary publishes the stores).
   if (bump && t == 0) {
-    __threadfence();
     const int32_t done = atomicAdd(ticket, 1);
     if (done == (int32_t)gridDim.x - 1) {
       *step_ptr = step;
