@@ -52,7 +52,12 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_int, c_int, c_int, c_int64, c_int, c_void_p, c_int, c_void_p,
          c_int64, c_int, c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p,
-         c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "da_topk_pages_lru": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_int, c_int, c_int, c_int64, c_int, c_void_p, c_int64,
+         c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p],
     ),
     "da_pages_gather": (
         c_int,

@@ -19,7 +19,7 @@
 // reference's literal serial walk on one lane per head.
 //
 // Bound: latency; algorithmic bytes are the metadata only.
-#include "select.hpp"
+#include "lru_keys.hpp"
 
 // Optional phase stamps for profiling builds (expands to nothing otherwise).
 #ifndef DA_LRU_STAMP
@@ -37,36 +37,6 @@ struct LruShared {
   uint32_t n_miss;
 };
 
-template <typename TimeT>
-__device__ __forceinline__ uint32_t time_order_key(TimeT v);
-template <>
-__device__ __forceinline__ uint32_t time_order_key<float>(float v) { return float_order_key(v); }
-template <>
-__device__ __forceinline__ uint32_t time_order_key<int32_t>(int32_t v) {
-  return (uint32_t)v ^ 0x80000000u;
-}
-
-// "largest key" = smallest access time, ties by lowest slot: the order of
-// torch.argsort(page_access_time, stable=True).
-template <typename TimeT>
-struct LeastRecentKey {
-  const TimeT *time;
-  __device__ __forceinline__ uint32_t operator()(int i) const {
-    return ~time_order_key<TimeT>(time[i]);
-  }
-  __device__ __forceinline__ void load4(int i, uint32_t *k) const {
-    TimeT v[4];
-    if (((uintptr_t)time & 15) == 0) {
-      *(u32x4 *)v = *(const u32x4 *)(time + i);
-    } else {
-#pragma unroll
-      for (int x = 0; x < 4; ++x) v[x] = time[i + x];
-    }
-#pragma unroll
-    for (int x = 0; x < 4; ++x) k[x] = ~time_order_key<TimeT>(v[x]);
-  }
-};
-
 __device__ __forceinline__ void atomic_min_signed(int32_t *p, int32_t v) { atomicMin(p, v); }
 __device__ __forceinline__ void atomic_min_signed(int64_t *p, int64_t v) {
   atomicMin((long long *)p, (long long)v);
@@ -82,7 +52,8 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
                   TimeT *time_all, int64_t time_head_stride, MapT *d2h_all,
                   int64_t d2h_head_stride, MapT *h2d_all, int64_t h2d_head_stride,
                   uint8_t *hit_mask, int32_t *miss_page_out, int32_t *miss_slot_out,
-                  int32_t *miss_count, int32_t *slot_epoch_all, int32_t *ticket, int serial) {
+                  int32_t *miss_count, int32_t *slot_epoch_all, int32_t *ticket, int serial,
+                  const int32_t *cand_all, int k_cand) {
   __shared__ LruShared sm;
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -191,7 +162,28 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
     DA_LRU_STAMP(2);
     // -- phase C: the m least recently used slots, in eviction order ---------
     const uint32_t *victims = nullptr;
-    if (m > 0) {
+    if (m > 0 && cand_all != nullptr && m <= k_cand) {
+      // The caller's list of the k_cand least recent slots, made before this call
+      // touched anything: untouched slots keep their order and still precede every
+      // touched one, so the first m untouched entries are the victims.
+      const int32_t slot = t < k_cand ? cand_all[(int64_t)h * k_cand + t] : 0;
+      const bool untouched = t < k_cand && time[slot] != now;
+      const uint64_t m_un = __ballot(untouched);
+      if (lane == 0) sm.wave_count[wave] = (uint32_t)__popcll(m_un);
+      __syncthreads();
+      uint32_t before = 0, total = 0;
+#pragma unroll
+      for (int w = 0; w < kSelWaves; ++w) {
+        const uint32_t c = sm.wave_count[w];
+        if (w < wave) before += c;
+        total += c;
+      }
+      const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+      if (untouched) sm.sel.idx_out[before + (uint32_t)__popcll(m_un & below)] = (uint32_t)slot;
+      __syncthreads();
+      if (total >= (uint32_t)m) victims = sm.sel.idx_out;  // else: too many were touched
+    }
+    if (m > 0 && victims == nullptr) {
       LeastRecentKey<TimeT> key{time};
       victims = select_sorted(key, n_hbm, m, sm.sel);
     }
@@ -262,16 +254,18 @@ static void launch_lru_time(int time_type, dim3 grid, hipStream_t s, const void 
                             int64_t idx_hs, int K, int64_t P, int n_hbm, int32_t *step, int bump,
                             void *time, int64_t time_hs, void *d2h, int64_t d2h_hs, void *h2d,
                             int64_t h2d_hs, uint8_t *hit, int32_t *mp, int32_t *ms, int32_t *mc,
-                            int32_t *se, int32_t *ticket, int serial) {
+                            int32_t *se, int32_t *ticket, int serial, const int32_t *cand,
+                            int k_cand) {
   if (time_type == DA_TIME_F32)
     hipLaunchKernelGGL((lru_update_kernel<IdxT, MapT, float>), grid, dim3(kSelThreads), 0, s,
                        (const IdxT *)idx, idx_hs, K, P, n_hbm, step, bump, (float *)time, time_hs,
-                       (MapT *)d2h, d2h_hs, (MapT *)h2d, h2d_hs, hit, mp, ms, mc, se, ticket, serial);
+                       (MapT *)d2h, d2h_hs, (MapT *)h2d, h2d_hs, hit, mp, ms, mc, se, ticket, serial,
+                       cand, k_cand);
   else
     hipLaunchKernelGGL((lru_update_kernel<IdxT, MapT, int32_t>), grid, dim3(kSelThreads), 0, s,
                        (const IdxT *)idx, idx_hs, K, P, n_hbm, step, bump, (int32_t *)time,
                        time_hs, (MapT *)d2h, d2h_hs, (MapT *)h2d, h2d_hs, hit, mp, ms, mc, se, ticket,
-                       serial);
+                       serial, cand, k_cand);
 }
 
 }  // namespace da
@@ -285,8 +279,11 @@ extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_i
                              int64_t d2h_head_stride, void *h2d, int64_t h2d_head_stride,
                              int map_itype, uint8_t *hit_mask, int32_t *miss_page,
                              int32_t *miss_slot, int32_t *miss_count, int32_t *slot_epoch,
-                             void *workspace, size_t workspace_bytes, void *stream) {
+                             const int32_t *candidates, int k_cand, void *workspace,
+                             size_t workspace_bytes, void *stream) {
   using namespace da;
+  DA_REQUIRE(k_cand >= 0 && k_cand <= kSelThreads && (k_cand == 0 || candidates != nullptr),
+             "da_lru_update: bad candidate list (%d entries, at most %d)", k_cand, kSelThreads);
   DA_REQUIRE(n_kv_heads >= 0 && k >= 0 && n_dram_pages >= 0 && n_hbm_pages >= 0,
              "da_lru_update: bad geometry (heads %d k %d pages %lld slots %d)", n_kv_heads, k,
              (long long)n_dram_pages, n_hbm_pages);
@@ -316,7 +313,8 @@ extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_i
 #define DA_LRU_ARGS                                                                          \
   time_type, grid, s, idx, idx_head_stride, k, n_dram_pages, n_hbm_pages, step, bump_step,   \
       access_time, time_head_stride, d2h, d2h_head_stride, h2d, h2d_head_stride, hit_mask,   \
-      miss_page, miss_slot, miss_count, slot_epoch, ticket, serial
+      miss_page, miss_slot, miss_count, slot_epoch, ticket, serial,                          \
+      (k_cand > 0 ? candidates : nullptr), k_cand
   if (idx_itype == DA_I64 && map_itype == DA_I64)
     launch_lru_time<int64_t, int64_t>(DA_LRU_ARGS);
   else if (idx_itype == DA_I64)

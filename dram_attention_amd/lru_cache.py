@@ -136,6 +136,7 @@ class LRUCache(torch.nn.Module):
 
         self._scratch = None
         self._topk_idx = None
+        self._have_candidates = False
 
     # -- internals ---------------------------------------------------------
     def _scratch_for(self, k: int) -> LruScratch:
@@ -143,6 +144,15 @@ class LRUCache(torch.nn.Module):
             self._scratch = LruScratch.allocate(self.num_kv_heads, k, self.hbm_kv_cache.device,
                                                 self.num_hbm_pages)
         return self._scratch
+
+    def _candidates_fit(self, idx: torch.Tensor) -> bool:
+        """Whether the list of least recently used slots that select_ left is current for
+        an update with ``idx``: it is for the request list select_ itself produced, once,
+        provided nothing updated the cache in between."""
+        use = (self._have_candidates and self._topk_idx is not None
+               and idx.data_ptr() == self._topk_idx.data_ptr() and idx.shape == self._topk_idx.shape)
+        self._have_candidates = False
+        return use
 
     def _views(self) -> CacheOutput:
         paged = self.hbm_kv_cache.view(
@@ -157,11 +167,12 @@ class LRUCache(torch.nn.Module):
         Advances ``current_step`` by one (inside the kernel, no host sync)."""
         if self._dram_device_ptr is None:
             self._dram_device_ptr = _lib.device_visible_ptr(self.dram_kv_cache)
+        scratch = self._scratch_for(top_k_dram_page_index.shape[1])
         lru_update_and_gather(
             self.dram_kv_cache, self.page_access_time, self.dram_page_to_hbm_page_mapping,
             self.hbm_page_to_dram_page_mapping, top_k_dram_page_index, self.current_step,
-            self.hbm_kv_cache, self._scratch_for(top_k_dram_page_index.shape[1]),
-            bump_step=True, dram_device_ptr=self._dram_device_ptr,
+            self.hbm_kv_cache, scratch, bump_step=True, dram_device_ptr=self._dram_device_ptr,
+            use_candidates=self._candidates_fit(top_k_dram_page_index),
         )
         return self._views()
 
@@ -185,14 +196,20 @@ class LRUCache(torch.nn.Module):
         if self._topk_idx is None or self._topk_idx.shape[1] != total:
             self._topk_idx = torch.empty(self.num_kv_heads, total, dtype=torch.int64,
                                          device=q.device)
-        return self.top_k_selector.top_k_for_lru(q, k, out=self._topk_idx)
+        # the same launch lists the least recently used slots for update_ (the
+        # order of the slots does not depend on the scores)
+        scratch = self._scratch_for(total)
+        self._have_candidates = True
+        return self.top_k_selector.top_k_for_lru(
+            q, k, out=self._topk_idx, lru=(self.page_access_time, scratch.candidates))
 
     def update_(self, idx: torch.Tensor) -> LruScratch:
         """Metadata only: advance the step, touch/evict/assign, emit the miss list."""
         scratch = self._scratch_for(idx.shape[1])
+        use = self._candidates_fit(idx)
         lru_update(self.dram_kv_cache, self.page_access_time, self.dram_page_to_hbm_page_mapping,
                    self.hbm_page_to_dram_page_mapping, idx, self.current_step, self.hbm_kv_cache,
-                   scratch, bump_step=True)
+                   scratch, bump_step=True, use_candidates=use)
         return scratch
 
     def gather_(self, k: int) -> None:

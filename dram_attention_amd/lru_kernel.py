@@ -22,6 +22,7 @@ class LruScratch(NamedTuple):
     hit_mask: torch.Tensor    # (H, K) uint8: 1 = resident when visited
     workspace: torch.Tensor   # zeroed once; holds the step-bump ticket
     slot_epoch: torch.Tensor  # (H, N_hbm) int32: step at which a slot was last re-assigned
+    candidates: torch.Tensor = None   # (H, k_cand) int32: least recent slots, when a selector fills it
 
     @staticmethod
     def allocate(num_heads: int, k: int, device, num_hbm_pages: int = 0) -> "LruScratch":
@@ -35,7 +36,12 @@ class LruScratch(NamedTuple):
             miss_count=torch.zeros(num_heads, dtype=torch.int32, device=device),
             hit_mask=torch.empty(num_heads, max(k, 1), dtype=torch.uint8, device=device),
             workspace=torch.zeros(ws, dtype=torch.uint8, device=device),
+            candidates=torch.empty(num_heads, max(min(num_hbm_pages, MAX_LRU_CANDIDATES), 1),
+                                   dtype=torch.int32, device=device),
         )
+
+
+MAX_LRU_CANDIDATES = 256  # least recent slots listed ahead of an update (one sort block's fast path)
 
 
 def lru_update(
@@ -49,10 +55,13 @@ def lru_update(
     scratch: LruScratch,
     bump_step: bool,
     serial_walk: bool = False,
+    use_candidates: bool = False,
 ) -> None:
     """The metadata half of a step: touch, evict, assign; leaves the miss list in
     ``scratch`` (one launch on the current stream).  ``serial_walk`` forces the
-    literal one-request-at-a-time walk (same result, for checks and baselines)."""
+    literal one-request-at-a-time walk (same result, for checks and baselines).
+    ``use_candidates``: ``scratch.candidates`` holds the least recently used slots
+    in eviction order as of right now (filled by ``topk_pages(..., lru=...)``)."""
     num_heads, num_dram_pages, page_dim = dram_kv_cache.shape
     _, k = topk_dram_page_index.shape
     assert (
@@ -93,11 +102,29 @@ def lru_update(
             scratch.hit_mask.data_ptr(), scratch.miss_page.data_ptr(),
             scratch.miss_slot.data_ptr(), scratch.miss_count.data_ptr(),
             epoch.data_ptr() if epoch is not None else None,
+            scratch.candidates.data_ptr() if use_candidates else None,
+            scratch.candidates.shape[1] if use_candidates else 0,
             scratch.workspace.data_ptr(), scratch.workspace.numel(),
             _lib.stream_ptr(hbm_kv_cache.device),
         ),
         "da_lru_update",
     )
+
+
+def lru_candidates(page_access_time: torch.Tensor, scratch: LruScratch) -> torch.Tensor:
+    """Fill ``scratch.candidates`` with the least recently used slots of every head, in
+    eviction order, as of now (one launch; normally this rides along with the top-k)."""
+    H, N = page_access_time.shape
+    cand = scratch.candidates
+    _lib.require_gpu(page_access_time, "page_access_time")
+    _lib.check(
+        _lib.load().da_topk_pages_lru(
+            None, 0, 0, 0, 1, H, 0, 0, None, 0, 0, 0, _lib.itype_code(torch.int64),
+            page_access_time.data_ptr(), page_access_time.stride(0),
+            _lib.time_code(page_access_time.dtype), N, cand.shape[1], cand.data_ptr(),
+            _lib.stream_ptr(page_access_time.device)),
+        "da_topk_pages_lru")
+    return cand
 
 
 def pages_gather(dram_kv_cache: torch.Tensor, hbm_kv_cache: torch.Tensor, scratch: LruScratch,
@@ -173,11 +200,12 @@ def lru_update_and_gather(
     bump_step: bool,
     dram_device_ptr: Optional[int] = None,
     serial_walk: bool = False,
+    use_candidates: bool = False,
 ) -> None:
     """Two launches on the current stream: metadata update, then page gather."""
     lru_update(dram_kv_cache, page_access_time, dram_page_to_hbm_page_mapping,
                hbm_page_to_dram_page_mapping, topk_dram_page_index, current_step, hbm_kv_cache,
-               scratch, bump_step, serial_walk)
+               scratch, bump_step, serial_walk, use_candidates)
     pages_gather(dram_kv_cache, hbm_kv_cache, scratch, topk_dram_page_index.shape[1],
                  dram_device_ptr)
 

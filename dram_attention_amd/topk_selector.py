@@ -35,17 +35,30 @@ def page_min_max(k_cache: torch.Tensor, num_pages: int) -> torch.Tensor:
 
 
 def topk_pages(scores: torch.Tensor, rep: int, k: int, out: torch.Tensor,
-               seq_stride: int, head_stride: int, rep_stride: int) -> torch.Tensor:
+               seq_stride: int, head_stride: int, rep_stride: int, lru=None) -> torch.Tensor:
     """Ordered top-k of every row of fp32 ``scores`` (n_rows, H, L); row n of head h
-    lands at (n // rep)*seq_stride + h*head_stride + (n % rep)*rep_stride in ``out``."""
+    lands at (n // rep)*seq_stride + h*head_stride + (n % rep)*rep_stride in ``out``.
+    ``lru`` = (page_access_time (H, N), candidates (H, k_cand) int32): the same launch
+    also lists the k_cand least recently used slots of every head, for the LRU
+    update that follows."""
     n_rows, H, L = scores.shape
     assert scores.dtype == torch.float32 and (L <= 1 or scores.stride(-1) == 1)
     lib = _lib.load()
+    if lru is None:
+        time_ptr, time_hs, time_code, n_slots, k_cand, cand_ptr = None, 0, 0, 0, 0, None
+    else:
+        access_time, candidates = lru
+        assert access_time.shape[0] == H and candidates.shape[0] == H
+        assert candidates.dtype == torch.int32 and candidates.is_contiguous()
+        time_ptr, time_hs = access_time.data_ptr(), access_time.stride(0)
+        time_code, n_slots = _lib.time_code(access_time.dtype), access_time.shape[1]
+        k_cand, cand_ptr = candidates.shape[1], candidates.data_ptr()
     _lib.check(
-        lib.da_topk_pages(
+        lib.da_topk_pages_lru(
             scores.data_ptr(), scores.stride(0), scores.stride(1), n_rows, rep, H, L, k,
             out.data_ptr(), seq_stride, head_stride, rep_stride, _lib.itype_code(out.dtype),
-            None, 0, _lib.stream_ptr(scores.device),
+            time_ptr, time_hs, time_code, n_slots, k_cand, cand_ptr,
+            _lib.stream_ptr(scores.device),
         ),
         "da_topk_pages",
     )
@@ -100,9 +113,10 @@ class IPUpperboundTopKSelector:
         out = torch.empty(seq_len, H, rep, k, dtype=torch.int64, device=q.device)
         return topk_pages(scores, rep, k, out, H * rep * k, rep * k, k)
 
-    def top_k_for_lru(self, q: torch.Tensor, k: int, out: torch.Tensor | None = None):
+    def top_k_for_lru(self, q: torch.Tensor, k: int, out: torch.Tensor | None = None, lru=None):
         """The same selection laid out as the LRU consumes it, (num_kv_heads,
-        seq_len*rep*k): what swapaxes(0,1).contiguous().view(H,-1) of top_k gives."""
+        seq_len*rep*k): what swapaxes(0,1).contiguous().view(H,-1) of top_k gives.
+        ``lru``: see :func:`topk_pages`."""
         bsz, seq_len, num_q_heads, _ = q.shape
         scores = self.scores(q)
         rep = num_q_heads // self.num_kv_heads
@@ -110,4 +124,4 @@ class IPUpperboundTopKSelector:
         k = min(k, L)
         if out is None:
             out = torch.empty(H, seq_len * rep * k, dtype=torch.int64, device=q.device)
-        return topk_pages(scores, rep, k, out, rep * k, seq_len * rep * k, k)
+        return topk_pages(scores, rep, k, out, rep * k, seq_len * rep * k, k, lru=lru)

@@ -130,6 +130,23 @@ int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
                   size_t workspace_bytes, void *stream);
 
 /*
+ * da_topk_pages, and in the same launch (one more workgroup per head) the list of
+ * the k_cand least recently used slots of every head, in eviction order, for the
+ * da_lru_update that follows (see its `candidates`).  The order of the slots
+ * does not depend on this step's scores, so it is computed next to the top-k
+ * instead of inside the LRU update, which every later launch of the step waits
+ * for.  Needs n_heads == Hkv; k_cand <= min(N_hbm, 1024); candidates == NULL or
+ * k_cand == 0 gives plain da_topk_pages.  n_rows == 0 or kp == 0 with a list
+ * requested computes the list only.
+ */
+int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_t head_stride,
+                      int n_rows, int rep, int n_heads, int64_t n_pages, int kp,
+                      void *out, int64_t out_seq_stride, int64_t out_head_stride,
+                      int64_t out_rep_stride, int out_itype, const void *access_time,
+                      int64_t time_head_stride, int time_type, int n_hbm_pages, int k_cand,
+                      int32_t *candidates, void *stream);
+
+/*
  * Subsystem 4a — LRU lookup / touch / evict / slot-assign for one decode step.
  * Replaces _update_page_access_time_, torch.argsort(page_access_time,
  * stable=True) and the metadata half of _load_lru_cache_inline_kernel in
@@ -143,6 +160,14 @@ int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
  *   hit_mask     : optional (Hkv, K) bytes, 1 = page was resident when visited
  *   miss_page/miss_slot : (Hkv, K) int32, the i-th distinct missed page of a
  *                  head and the slot it was given; miss_count : (Hkv) int32
+ *   candidates   : optional (Hkv, k_cand) int32 from da_topk_pages_lru: the k_cand
+ *                  least recently used slots of every head in eviction order, taken
+ *                  after the previous da_lru_update and before this one.  The
+ *                  kernel then finds its victims by dropping the slots this call
+ *                  touches from that list instead of ordering all slots again (it
+ *                  orders them itself whenever the list is too short); a list
+ *                  that does not describe the current access times gives wrong
+ *                  evictions.  NULL / k_cand = 0: no list.
  *   slot_epoch   : optional (Hkv, N_hbm) int32; a slot handed to a missed page
  *                  gets the step value, so a later kernel can tell which slots
  *                  the page stream of this step is (still) writing
@@ -167,7 +192,8 @@ int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_itype,
                   int64_t d2h_head_stride, void *h2d, int64_t h2d_head_stride,
                   int map_itype, uint8_t *hit_mask, int32_t *miss_page,
                   int32_t *miss_slot, int32_t *miss_count, int32_t *slot_epoch,
-                  void *workspace, size_t workspace_bytes, void *stream);
+                  const int32_t *candidates, int k_cand, void *workspace,
+                  size_t workspace_bytes, void *stream);
 
 /*
  * Subsystem 4b — stream the missed pages into their HBM slots.

@@ -234,10 +234,10 @@ def test_load_lru_cache_reference_kats(name):
 
 
 def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat16, page_dim=256,
-              hot=None, serial_walk=False):
+              hot=None, serial_walk=False, candidates=False):
     """Random request trace on LRUCache-like state; compares every buffer with the
     oracle's serial walk after every step."""
-    from dram_attention_amd.lru_kernel import LruScratch, lru_update_and_gather
+    from dram_attention_amd.lru_kernel import LruScratch, lru_candidates, lru_update_and_gather
 
     rng = np.random.default_rng(seed)
     dram = torch.randn(H, P, page_dim, generator=gen(seed)).to(dtype)
@@ -249,7 +249,7 @@ def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat1
     d2h = torch.from_numpy(st.d2h).to(itype).to(DEV)
     h2d = torch.from_numpy(st.h2d).to(itype).to(DEV)
     step = torch.zeros(1, dtype=torch.int32, device=DEV)
-    scratch = LruScratch.allocate(H, K, DEV)
+    scratch = LruScratch.allocate(H, K, DEV, N)
     as_np = (lambda t: t.view(torch.int16).numpy()) if dtype != torch.float32 else (lambda t: t.numpy())
     for s in range(1, steps + 1):
         if hot:  # skewed requests with duplicates, like overlapping per-head top-k lists
@@ -258,8 +258,13 @@ def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat1
         else:
             idx = rng.integers(0, P, (H, K))
         hit_o, miss_o = O.lru_load(st, idx, s, as_np(dram), as_np(hbm_o))
+        if candidates:   # the least recent slots listed ahead of the update, as the module does
+            order = lru_candidates(time, scratch).cpu()
+            want = torch.sort(time.cpu().float(), dim=1, stable=True).indices[:, :order.shape[1]]
+            assert same(order.long(), want), f"candidates, step {s}"
         lru_update_and_gather(dram_dev, time, d2h, h2d, torch.from_numpy(idx).to(itype).to(DEV),
-                              step, hbm, scratch, bump_step=True, serial_walk=serial_walk)
+                              step, hbm, scratch, bump_step=True, serial_walk=serial_walk,
+                              use_candidates=candidates)
         torch.cuda.synchronize()
         assert step.item() == s
         assert np.array_equal(time.cpu().numpy().astype(np.float32), st.time), f"time, step {s}"
@@ -292,6 +297,20 @@ def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat1
 def test_lru_update_matches_serial_walk(H, P, N, K, itype, ttype, pinned):
     lru_trace(H, P, N, K, 12, 100 + K, itype, ttype, pinned)
     lru_trace(H, P, N, K, 12, 200 + K, itype, ttype, pinned, hot=max(2, P // 8))
+
+
+@pytest.mark.parametrize("H,P,N,K,ttype", [
+    (8, 8192, 2048, 1024, torch.float32),     # the 128K layer: list of 512, ~120 victims per step
+    (4, 1024, 256, 200, torch.float32),       # list of 256 with up to 200 of them touched: falls back
+    (2, 4096, 600, 64, torch.int32),          # list of 512 of 600 slots
+    (3, 300, 100, 37, torch.float32),
+])
+def test_lru_update_with_candidate_list_matches_serial_walk(H, P, N, K, ttype):
+    """Victims taken from the list of least recent slots made ahead of the update
+    (touched ones dropped), with the kernel's own ordering as the fallback."""
+    lru_trace(H, P, N, K, 10, 400 + K, torch.int64, ttype, False, candidates=True)
+    lru_trace(H, P, N, K, 10, 500 + K, torch.int64, ttype, False, hot=max(2, P // 8),
+              candidates=True)
 
 
 def test_lru_update_forced_serial_walk_gives_the_same_state():
