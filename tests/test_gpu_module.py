@@ -189,6 +189,36 @@ def test_module_prefill_then_generate_shapes():
     assert o1.shape == (1, 1, 32, 128) and torch.isfinite(o1.float()).all()
 
 
+def test_prefill_call_then_generate_matches_oracle():
+    """The model-side sequence of the reference (forward with stage="prefill" and
+    start_pos=0, then one generate call per token with integer positions): the cache
+    the prefill call builds decodes like the oracle's built from the same K/V."""
+    from dram_attention_amd import DRAMAttention, LRUCache
+
+    w = WORKLOADS["128k"].scaled(dram_tokens=8192, local_cache=512, lru_tokens=2048,
+                                 top_k_tokens=512, steps=4)
+    prompt = make_prompt(w, 21)
+    S = w.prompt_tokens
+    g = torch.Generator().manual_seed(22)
+    xq0 = torch.randn(1, S, w.n_q_heads, w.head_dim, generator=g).to(w.dtype)
+    m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                      w.n_kv_heads, w.head_dim, device=DEV, dtype=w.dtype)
+    out0 = m(xq0.to(DEV), prompt.k.to(DEV), prompt.v.to(DEV), start_pos=0, stage="prefill")
+    assert out0.shape == xq0.shape and isinstance(m.lru_cache, LRUCache)
+    o = O.DecodeOracle(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                       w.n_kv_heads, w.head_dim, dtype=w.dtype)
+    o.init_cache(prompt.k, prompt.v)
+    assert m.dram_kv_cache_size == o.dram_kv_cache_size
+    assert same(m.lru_cache.dram_kv_cache, o.dram)
+    inputs = DecodeInputs(w, prompt.q0, 21)
+    for t in range(w.steps):
+        xq, xk, xv = inputs.next()
+        got = m(xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=S + t, stage="generate")
+        want = o.generate(xq, xk, xv, S + t, scores=m.lru_cache.top_k_selector._scores.cpu())
+        assert same(m.lru_cache._topk_idx.cpu(), o.last_idx)
+        assert close(got.cpu().float(), want.float(), 2e-2, 1e-2), f"step {t}"
+
+
 # ------------------------------------------------------------ whole decode runs vs the oracle
 def run_parity(w, seed, steps, atol, rtol, device_pos=False):
     """Drives the module and the oracle with the same inputs.  Selection and LRU
