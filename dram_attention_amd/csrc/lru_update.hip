@@ -101,6 +101,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
           d2h[p] = (MapT)v;
           mpage[m] = (int32_t)p;
           mslot[m] = v;
+          sm.miss_page[v] = m;  // the latest entry that targets slot v (n_hbm <= kLruMaxK here)
           if (slot_epoch) slot_epoch[v] = step;
           ++m;
           ep = ep + 1 == n_hbm ? 0 : ep + 1;
@@ -114,10 +115,13 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       miss_count[h] = m;
     }
     __syncthreads();
-    // an entry whose slot was handed out again later in the walk is dead
+    // Only the last entry that targets a slot is live: the slot may have been handed
+    // out again later in the walk, to another page or to the same page once more
+    // (evicted and requested again), and a consumer that walks the list must meet
+    // every slot once.
     const int m = (int)sm.n_miss;
     for (int i = t; i < m; i += kSelThreads)
-      if ((int64_t)h2d[mslot[i]] != (int64_t)mpage[i]) mslot[i] = -1;
+      if (sm.miss_page[mslot[i]] != i) mslot[i] = -1;
   } else {
     // -- phase A: touch hits, mark the first occurrence of every missed page --
     for (int k = t; k < K; k += kSelThreads) {

@@ -278,12 +278,14 @@ def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat1
             got = [(int(mp[h, i]), int(ms[h, i])) for i in range(counts[h])]
             if K <= N:
                 assert got == miss_o[h]
-            else:  # serial walk: entries overwritten later in the call are marked dead
-                live = {}
-                for p, v in miss_o[h]:
-                    live[v] = p
+            else:  # serial walk: only the last entry that targets a slot stays live
+                last = {}
+                for i, (p, v) in enumerate(miss_o[h]):
+                    last[v] = i
                 assert [(p, v) for p, v in got if v >= 0] == \
-                    [(p, v) for p, v in miss_o[h] if live[v] == p]
+                    [(p, v) for i, (p, v) in enumerate(miss_o[h]) if last[v] == i]
+                live_slots = [v for p, v in got if v >= 0]
+                assert len(live_slots) == len(set(live_slots))
         assert same(hbm.cpu(), hbm_o), f"payload, step {s}"
 
 
@@ -319,10 +321,14 @@ def test_lru_update_forced_serial_walk_gives_the_same_state():
     lru_trace(2, 512, 128, 128, 6, 78, torch.int32, torch.int32, True, hot=64, serial_walk=True)
 
 
-@pytest.mark.parametrize("H,P,N,K", [(2, 40, 6, 17), (1, 8, 2, 3), (3, 200, 50, 120)])
+@pytest.mark.parametrize("H,P,N,K", [(2, 40, 6, 17), (1, 8, 2, 3), (3, 200, 50, 120),
+                                     (2, 60, 10, 70)])
 def test_lru_update_more_requests_than_slots(H, P, N, K):
     lru_trace(H, P, N, K, 8, 300 + K, torch.int64, torch.float32, False, dtype=torch.float32,
               page_dim=32)
+    # requests crowded onto few pages: a page comes back to the slot it was evicted from
+    lru_trace(H, P, N, K, 8, 350 + K, torch.int64, torch.float32, False, dtype=torch.float32,
+              page_dim=32, hot=max(3, N + 2))
     lru_trace(H, P, N, K, 8, 400 + K, torch.int64, torch.float32, False, dtype=torch.float32,
               page_dim=32, hot=max(2, P // 4))
 

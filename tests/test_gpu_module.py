@@ -337,6 +337,32 @@ def test_decode_parity_long_run_with_heavy_eviction():
     assert rate < 0.95      # the run really paged
 
 
+def random_small_workload(rng):
+    dtype = [torch.bfloat16, torch.float16, torch.float32][rng.integers(0, 3)]
+    head_dim = int(rng.choice([64, 128] if dtype != torch.float32 else [32, 64]))
+    n_kv = int(rng.integers(1, 5))
+    rep = int(rng.choice([1, 2, 3, 4, 7, 8]))
+    page = int(rng.choice([8, 16, 32]))
+    n_pages = int(rng.integers(40, 200))
+    n_slots = int(rng.integers(8, n_pages // 2))
+    kp = int(rng.integers(1, min(n_slots, 24) + 1))
+    local_pages = int(rng.integers(1, 9))
+    return WORKLOADS["128k"].scaled(
+        dtype=dtype, n_q_heads=n_kv * rep, n_kv_heads=n_kv, head_dim=head_dim, page_size=page,
+        dram_tokens=n_pages * page, local_cache=local_pages * page, lru_tokens=n_slots * page,
+        top_k_tokens=kp * page, steps=3)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_decode_parity_random_small_shapes(seed):
+    """Seeded sweep over head counts, GQA widths (also 3 and 7), head sizes, page sizes,
+    cache geometries with more or fewer requests than slots, and the three dtypes."""
+    rng = np.random.default_rng(1000 + seed)
+    w = random_small_workload(rng)
+    tol = {torch.float32: (1e-4, 1e-4), torch.float16: (4e-3, 1e-2), torch.bfloat16: (2e-2, 1e-2)}
+    run_parity(w, 100 + seed, w.steps, *tol[w.dtype])
+
+
 def test_page_stream_overlap_changes_nothing():
     """Attention issued around a concurrent page stream (two phases, side stream)
     gives the bits of the serialised order, and both agree with one plain pass."""
