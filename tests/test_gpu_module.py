@@ -363,6 +363,38 @@ def test_decode_parity_random_small_shapes(seed):
     run_parity(w, 100 + seed, w.steps, *tol[w.dtype])
 
 
+@pytest.mark.parametrize("seed", range(32))
+def test_stream_variants_agree_on_random_small_shapes(seed):
+    """Same workload through the three ways of running the page stream: inside the
+    attention launch, as its own launch before attention (same bits), and copy-only
+    with a tail pass (same state, output equal up to the merge order)."""
+    from dram_attention_amd import DRAMAttention
+
+    rng = np.random.default_rng(6000 + seed)
+    w = random_small_workload(rng)
+    prompt = make_prompt(w, 200 + seed)
+    mods = []
+    for overlap, fused in ((True, True), (False, True), (True, False)):
+        m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                          w.n_kv_heads, w.head_dim, device=DEV, dtype=w.dtype)
+        m.overlap_page_stream, m.attend_on_page_stream = overlap, fused
+        m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+        mods.append(m)
+    inputs = DecodeInputs(w, prompt.q0, 200 + seed)
+    atol, rtol = {torch.float32: (1e-5, 1e-4), torch.float16: (2e-3, 1e-2),
+                  torch.bfloat16: (1e-2, 1e-2)}[w.dtype]
+    for t in range(w.steps):
+        xq, xk, xv = (x.to(DEV) for x in inputs.next())
+        outs = [m(xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate") for m in mods]
+        torch.cuda.synchronize()
+        assert same(outs[0], outs[1]), f"step {t}"
+        assert close(outs[0].float(), outs[2].float(), atol, rtol), f"step {t}"
+        for m in mods[1:]:
+            assert same(m.lru_cache.hbm_kv_cache, mods[0].lru_cache.hbm_kv_cache)
+            assert same(m.lru_cache.page_access_time, mods[0].lru_cache.page_access_time)
+            assert same(m.cache_k, mods[0].cache_k)
+
+
 def test_page_stream_overlap_changes_nothing():
     """Attention issued around a concurrent page stream (two phases, side stream)
     gives the bits of the serialised order, and both agree with one plain pass."""
