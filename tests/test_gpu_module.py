@@ -475,7 +475,8 @@ def test_attention_on_the_page_stream_equals_tail_pass(base, kw):
     assert misses > 0
 
 
-def test_graph_replay_equals_eager_steps():
+@pytest.mark.parametrize("fused", [True, False])
+def test_graph_replay_equals_eager_steps(fused):
     """The whole step (selection, LRU, page stream on its side stream, two-phase
     attention, append) captured once and replayed: every replay, with eager work
     and synchronisations in between, gives the eager module's bits and state."""
@@ -488,6 +489,7 @@ def test_graph_replay_equals_eager_steps():
     for _ in range(2):
         m = DRAMAttention(w.steps + 1, w.lru_tokens, w.local_cache, 16, w.top_k_tokens, w.n_kv_heads,
                           w.head_dim, device=DEV, dtype=w.dtype)
+        m.attend_on_page_stream = fused   # False: page stream on a side stream, fork/join captured
         m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
         mods.append(m)
     graphed, eager = mods
