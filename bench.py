@@ -555,6 +555,9 @@ def main():
             "algorithmic_bytes": attn_b, "avg_us": attn_us,
         },
         "kernels_us": kernel_us,
+        "kernels_us_note": "events around 8 back-to-back launches per kernel, except lru_update: it "
+                           "changes its own input, so it is one launch and ~4 us of launch latency "
+                           "sit inside its figure (its kernel time in the profiler is ~9 us)",
         "page_score_GBps": score_gbps,
         "page_stream": {"requests_per_step": requests, "distinct_misses_per_step": miss_per_step,
                         "h2d_bytes_per_step": miss_per_step * page_bytes,
