@@ -52,6 +52,9 @@ def parse_args():
                     help="attention layers per model step, each with its own page cache and inputs "
                          "(seed + layer); 32 with workload 128k is configs[3].  One model step per "
                          "graph; value stays per layer: layer-steps per second")
+    ap.add_argument("--force-lru", action="store_true",
+                    help="workload 32k: run the page-cache path although the prefix fits the cache "
+                         "(every request hits; the reference's init_cache would pick the static cache)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-steps", type=int, default=64, help="steps of the CPU oracle to time (0 = skip)")
     ap.add_argument("--reference-shaped-steps", type=int, default=24,
@@ -65,8 +68,8 @@ def parse_args():
 class Layer:
     """One attention layer set up on the workload, plus the staged step inputs."""
 
-    def __init__(self, w, seed, total_steps, dev, overlap):
-        from dram_attention_amd import DRAMAttention
+    def __init__(self, w, seed, total_steps, dev, overlap, force_lru=False):
+        from dram_attention_amd import DRAMAttention, DummyCache, LRUCache
         from dram_attention_amd.synthetic import DecodeInputs, make_prompt
 
         self.w = w
@@ -78,6 +81,14 @@ class Layer:
                                device=dev, dtype=w.dtype)
         self.m.overlap_page_stream = overlap
         self.m.init_cache(prompt.k.to(dev), prompt.v.to(dev))
+        if force_lru and isinstance(self.m.lru_cache, DummyCache):
+            # the prefix fits the page cache, so init_cache chose the static cache; a page
+            # cache built directly over the same prefix is the all-hits point of the LRU path
+            S = self.m.dram_kv_cache_size
+            self.m.lru_cache = LRUCache(prompt.k[0, :S].to(dev).transpose(0, 1),
+                                        prompt.v[0, :S].to(dev).transpose(0, 1), w.page_size,
+                                        w.top_k_tokens // w.page_size, w.lru_tokens, device=dev)
+            self.m._workspace = None
         inputs = DecodeInputs(w, prompt.q0, seed)
         qs, ks, vs = zip(*(inputs.next() for _ in range(total_steps)))
         self.host_inputs = (qs, ks, vs)
@@ -444,7 +455,8 @@ def main():
     total = args.warmup + args.steps + args.profile_steps + 4
     layers = []
     for li in range(max(args.layers, 1)):
-        layers.append(Layer(w, args.seed + li, total, dev, overlap=not args.no_overlap))
+        layers.append(Layer(w, args.seed + li, total, dev, overlap=not args.no_overlap,
+                            force_lru=args.force_lru))
         if li > 0:
             layers[-1].prompt = None   # only layer 0 feeds the CPU baseline
         if args.layers > 1:
@@ -547,6 +559,7 @@ def main():
             "model_steps_per_s": args.steps / dt,
             "page_stream": "serialised" if args.no_overlap else "in the launch of the first attention pass",
             "seed": args.seed,
+            "cache": type(layer.m.lru_cache).__name__,
         },
         "roofline": {
             "bound": "hbm", "kernel": "decode_attention_split_kernel (prefix + local segments)",
