@@ -23,6 +23,7 @@ SOURCES = (
     "topk_pages.hip",
     "lru_update.hip",
     "decode_attention.hip",
+    "stream_attention.hip",
 )
 # packed fp32 VALU ops are switched off for every device compile of this library
 HIPCC_FLAGS = (

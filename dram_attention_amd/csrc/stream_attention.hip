@@ -1,0 +1,167 @@
+// Launches that carry the page stream: the attending stream alone
+// (da_pages_gather_attend) and the stream plus the first attention pass in one
+// grid (what da_decode_attention_paged issues for DA_PHASE_STREAM).  Neither
+// has a counterpart in the reference, which copies pages with index_select /
+// index_copy_ (dram_attention/lru_cache.py:224-241) before it attends.
+#include "page_stream.hpp"
+
+namespace da {
+
+template <typename T, int kLanes, int kRows>
+__global__ void __launch_bounds__(kGatherThreads)
+pages_gather_attend_kernel(const GatherAttendArgs g) {
+  gather_attend_block<T, kLanes, kRows>(g, blockIdx.y * gridDim.x + blockIdx.x,
+                                        gridDim.x * gridDim.y);
+}
+
+// Both of the above in one launch: blocks [0, g_blocks) of every kv head run the
+// page stream, the others the first attention pass (prefix minus the slots under
+// rewrite, plus the local segment).  One kernel instead of two on two streams
+// keeps the step a plain chain of launches: no fork and join around the long
+// pole of the step, each of which costs about 5 us of dependency latency.
+static_assert(kGatherThreads == kAttnThreads, "one block shape for both roles");
+template <typename T, int kLanes, int kRowsAttn, int kRowsGather>
+__global__ void __launch_bounds__(kAttnThreads)
+decode_stream_attend_kernel(const AttnArgs a, const GatherAttendArgs g, const int g_blocks) {
+  if ((int)blockIdx.x < g_blocks) {
+    if (blockIdx.z == 0)
+      gather_attend_block<T, kLanes, kRowsGather>(g, blockIdx.y * g_blocks + blockIdx.x,
+                                                  g_blocks * gridDim.y);
+  } else {
+    attention_split_block<T, kLanes, kRowsAttn, false>(a, (int)blockIdx.x - g_blocks);
+  }
+}
+
+// The page stream and the first attention pass as one launch.
+template <typename T, int kLanes>
+static void launch_stream_attend(AttnArgs a, const GatherAttendArgs &g, int g_blocks, int n_chunks,
+                                 int n_kv_heads, hipStream_t s) {
+  a.chunk_base = 0;
+  const int rep = a.rep;
+  if (rep > 4 && kLanes <= 16) {
+    const dim3 grid(g_blocks + n_chunks, n_kv_heads, 1);
+    hipLaunchKernelGGL((decode_stream_attend_kernel<T, (kLanes <= 16 ? kLanes : 16), 8, 8>), grid,
+                       dim3(kAttnThreads), 0, s, a, g, g_blocks);
+  } else {
+    const dim3 grid(g_blocks + n_chunks, n_kv_heads, (unsigned)ceil_div(rep, 4));
+    if (rep > 4)
+      hipLaunchKernelGGL((decode_stream_attend_kernel<T, kLanes, 4, 8>), grid, dim3(kAttnThreads),
+                         0, s, a, g, g_blocks);
+    else
+      hipLaunchKernelGGL((decode_stream_attend_kernel<T, kLanes, 4, 4>), grid, dim3(kAttnThreads),
+                         0, s, a, g, g_blocks);
+  }
+}
+
+template <typename T>
+static int dispatch_stream_attend(const AttnArgs &a, const GatherAttendArgs &g, int lanes,
+                                  int n_chunks, int n_kv_heads, hipStream_t s) {
+  switch (lanes) {
+    case 4: launch_stream_attend<T, 4>(a, g, a.gather_blocks, n_chunks, n_kv_heads, s); break;
+    case 8: launch_stream_attend<T, 8>(a, g, a.gather_blocks, n_chunks, n_kv_heads, s); break;
+    case 16: launch_stream_attend<T, 16>(a, g, a.gather_blocks, n_chunks, n_kv_heads, s); break;
+    case 32: launch_stream_attend<T, 32>(a, g, a.gather_blocks, n_chunks, n_kv_heads, s); break;
+    default: return fail(DA_ENOTSUP, "page stream with attention: rows of %d bytes", lanes * 16);
+  }
+  return launch_status("da_decode_attention(page stream + first pass)");
+}
+
+int launch_stream_attend(const AttnArgs &a, const GatherAttendArgs &g, int dtype, int lanes,
+                         int n_chunks, int n_kv_heads, hipStream_t s) {
+  switch (dtype) {
+    case DA_F32: return dispatch_stream_attend<F32>(a, g, lanes, n_chunks, n_kv_heads, s);
+    case DA_F16: return dispatch_stream_attend<F16>(a, g, lanes, n_chunks, n_kv_heads, s);
+    default: return dispatch_stream_attend<BF16>(a, g, lanes, n_chunks, n_kv_heads, s);
+  }
+}
+
+template <typename T, int kLanes>
+static void launch_gather_attend(const GatherAttendArgs &g, dim3 grid, hipStream_t s) {
+  if (g.rep <= 4)
+    hipLaunchKernelGGL((pages_gather_attend_kernel<T, kLanes, 4>), grid, dim3(kGatherThreads), 0, s,
+                       g);
+  else
+    hipLaunchKernelGGL((pages_gather_attend_kernel<T, kLanes, 8>), grid, dim3(kGatherThreads), 0, s,
+                       g);
+}
+
+template <typename T>
+static int dispatch_gather_attend(const GatherAttendArgs &g, int lanes, dim3 grid, hipStream_t s) {
+  switch (lanes) {
+    case 4: launch_gather_attend<T, 4>(g, grid, s); break;
+    case 8: launch_gather_attend<T, 8>(g, grid, s); break;
+    case 16: launch_gather_attend<T, 16>(g, grid, s); break;
+    case 32: launch_gather_attend<T, 32>(g, grid, s); break;
+    default: return fail(DA_ENOTSUP, "da_pages_gather_attend: rows of %d bytes", lanes * 16);
+  }
+  return launch_status("da_pages_gather_attend");
+}
+
+}  // namespace da
+
+extern "C" int da_pages_gather_attend(
+    const void *dram, int64_t dram_head_stride_bytes, int64_t dram_page_stride_bytes, void *hbm,
+    int64_t hbm_head_stride_bytes, int64_t hbm_slot_stride_bytes, int page_size,
+    const int32_t *miss_page, const int32_t *miss_slot, const int32_t *miss_count, int n_kv_heads,
+    int k, int blocks_per_head, const void *q, int64_t q_head_stride, int n_q_heads, int head_dim,
+    int dtype, float scale, int64_t p_len, int64_t c_capacity, void *workspace,
+    size_t workspace_bytes, void *stream) {
+  using namespace da;
+  DA_REQUIRE(n_kv_heads > 0 && n_q_heads > 0 && n_q_heads % n_kv_heads == 0 && k > 0 &&
+                 page_size > 0 && p_len >= 0 && c_capacity >= 0,
+             "da_pages_gather_attend: bad geometry");
+  DA_REQUIRE(dtype == DA_F32 || dtype == DA_F16 || dtype == DA_BF16,
+             "da_pages_gather_attend: unknown dtype %d", dtype);
+  DA_REQUIRE(dram && hbm && miss_page && miss_slot && miss_count && q && workspace,
+             "da_pages_gather_attend: null pointer");
+  DA_REQUIRE(blocks_per_head >= 1 && (int64_t)blocks_per_head * n_kv_heads <= kGatherMaxBlocks,
+             "da_pages_gather_attend: blocks_per_head %d x %d kv heads not in 1..%d",
+             blocks_per_head, n_kv_heads, kGatherMaxBlocks);
+  const int lanes = lanes_of(head_dim, dtype);
+  const int rep = n_q_heads / n_kv_heads;
+  const int64_t page_vecs = (int64_t)page_size * 2 * lanes;
+  if (!lanes || lanes > 32 || rep > 8 || page_vecs > kGatherThreads * kGatherMaxLoads ||
+      n_kv_heads > 65535)
+    return fail(DA_ENOTSUP,
+                "da_pages_gather_attend: needs rows of 64..512 bytes, at most 8 query heads per kv "
+                "head and pages up to %d bytes (use da_pages_gather and the tail pass instead)",
+                kGatherThreads * kGatherMaxLoads * 16);
+  const int vec = dtype == DA_F32 ? 4 : 8;
+  DA_REQUIRE(dram_head_stride_bytes % 16 == 0 && dram_page_stride_bytes % 16 == 0 &&
+                 hbm_head_stride_bytes % 16 == 0 && hbm_slot_stride_bytes % 16 == 0 &&
+                 (uintptr_t)dram % 16 == 0 && (uintptr_t)hbm % 16 == 0 && (uintptr_t)q % 16 == 0 &&
+                 q_head_stride % vec == 0 && (uintptr_t)workspace % 16 == 0,
+             "da_pages_gather_attend: operands must be 16-byte aligned");
+  const ChunkPlan p = plan_chunks(n_kv_heads, lanes, p_len, c_capacity, (int64_t)k * page_size);
+  const size_t need = attn_workspace_bytes(n_q_heads, head_dim, p.total());
+  DA_REQUIRE(workspace_bytes >= need, "da_pages_gather_attend: workspace %zu < %zu bytes",
+             workspace_bytes, need);
+  GatherAttendArgs g = {};
+  g.dram = (const char *)dram;
+  g.dram_head_stride = dram_head_stride_bytes;
+  g.dram_page_stride = dram_page_stride_bytes;
+  g.hbm = (char *)hbm;
+  g.hbm_head_stride = hbm_head_stride_bytes;
+  g.hbm_slot_stride = hbm_slot_stride_bytes;
+  g.page_vecs = (int)page_vecs;
+  g.miss_page = miss_page;
+  g.miss_slot = miss_slot;
+  g.miss_count = miss_count;
+  g.K = k;
+  g.q = (const char *)q;
+  g.q_head_stride = q_head_stride;
+  g.rep = rep;
+  g.n_q_heads = n_q_heads;
+  g.n_kv_heads = n_kv_heads;
+  g.scale_log2 = scale * kLog2e;
+  g.part_acc = (float *)workspace;
+  g.part_ml = g.part_acc + (size_t)p.total() * n_q_heads * head_dim;
+  g.chunk0 = p.gather_chunk0();
+  const dim3 grid(blocks_per_head, n_kv_heads);
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case DA_F32: return dispatch_gather_attend<F32>(g, lanes, grid, s);
+    case DA_F16: return dispatch_gather_attend<F16>(g, lanes, grid, s);
+    default: return dispatch_gather_attend<BF16>(g, lanes, grid, s);
+  }
+}
