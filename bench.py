@@ -60,6 +60,10 @@ def parse_args():
     ap.add_argument("--reference-shaped-steps", type=int, default=24,
                     help="steps of the reference-shaped stand-in pipeline to time (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=16, help="extra steps timed per kernel with events")
+    ap.add_argument("--model-decode-steps", type=int, default=0,
+                    help="also time greedy decoding of a Llama-3.1-8B-shaped model (random weights, "
+                         "random K/V of the workload's prompt length in every layer's page cache), "
+                         "whole model step per HIP graph; 0 = skip")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 128 MiB device copy (reference point for HBM traffic counters)")
     return ap.parse_args()
@@ -432,6 +436,46 @@ def reference_shaped(w, seed, steps, dev):
                     "and one-workgroup-per-head page copy for its Triton stages; launched eagerly (GPU-bound)"}
 
 
+def model_decode(w, steps, seed, dev):
+    """Tokens per second of a Llama-3.1-8B-shaped decoder (32 layers, random bf16
+    weights) whose every layer holds a page cache over a random prompt of the
+    workload's length: the figure the reference's chat example prints, with the
+    model step captured in one graph as it does."""
+    from dram_attention_amd.llama import GraphedDecoder, ModelArgs, Transformer
+
+    torch.manual_seed(seed)
+    a = ModelArgs(dim=w.n_q_heads * w.head_dim, n_layers=32, n_heads=w.n_q_heads,
+                  n_kv_heads=w.n_kv_heads, vocab_size=128256, multiple_of=1024,
+                  ffn_dim_multiplier=1.3, rope_theta=500000.0, use_scaled_rope=True,
+                  lru_hbm_cache_size=w.lru_tokens, local_cache_size=w.local_cache,
+                  cache_page_size=w.page_size, cache_top_k=w.top_k_tokens,
+                  max_output_length=steps + 8, max_seq_len=w.prompt_tokens + steps + 8,
+                  dtype=w.dtype)
+    model = Transformer(a, device=dev)
+    shape = (1, w.prompt_tokens, w.n_kv_heads, w.head_dim)
+    for layer in model.layers:
+        k = torch.randn(shape, device=dev, dtype=w.dtype)
+        v = torch.randn(shape, device=dev, dtype=w.dtype)
+        layer.attention.dram_attention.init_cache(k, v)
+        del k, v
+    dec = GraphedDecoder(model, w.prompt_tokens, first_token=1)
+    dec.step()                       # eager: sizes the workspaces
+    dec.step()                       # captures the graph and replays it once
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        dec.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    misses = sum(l_.attention.dram_attention.lru_cache.last_miss_counts().sum().item()
+                 for l_ in model.layers) / a.n_layers
+    params = sum(p.numel() for p in model.parameters())
+    return {"value": steps / dt, "unit": "tokens/s", "ms_per_token": dt / steps * 1e3,
+            "steps": steps, "model": "Llama-3.1-8B shape, random weights", "parameters": params,
+            "prompt_tokens": w.prompt_tokens, "distinct_misses_per_layer_last_step": misses,
+            "launch": "one HIP graph per token (32 layers)"}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -601,6 +645,10 @@ def main():
             return ref
 
         leg("reference_shaped_gpu", ref_leg)
+    if args.model_decode_steps > 0:
+        layer = layers = model_step = None
+        torch.cuda.empty_cache()
+        leg("model_decode", lambda: model_decode(w, args.model_decode_steps, args.seed, dev))
     print(json.dumps(result))
     return 0
 
