@@ -4,9 +4,6 @@
 // and by the launch that also carries the page stream (stream_attention.hip).
 #pragma once
 #include "common.hpp"
-#ifdef DA_TUNE
-#include <stdlib.h>
-#endif
 
 namespace da {
 
@@ -20,10 +17,7 @@ constexpr float kMinusHuge = -1.0e30f;  // finite stand-in for -inf as a running
 constexpr float kRescaleSlack = 8.0f;
 constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = kAttnThreads / 64;
-#ifndef DA_ATTN_UNROLL
-#define DA_ATTN_UNROLL 4
-#endif
-constexpr int kAttnUnroll = DA_ATTN_UNROLL;  // tokens in flight per lane group (even)
+constexpr int kAttnUnroll = 4;  // tokens in flight per lane group (even)
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -411,10 +405,7 @@ inline int pick_chunk(int64_t total_tokens, int n_kv_heads, int step_tokens) {
   // merge epilogue, so few long chunks beat many short ones (measured on the
   // 128K workload: 31.9 us at 512 blocks, 32.6 us at 2048); never below one
   // unrolled round.
-  int64_t want_blocks = 256 * 2;
-#ifdef DA_TUNE
-  if (const char *e = getenv("DA_ATTN_BLOCKS")) want_blocks = atoi(e);
-#endif
+  const int64_t want_blocks = 256 * 2;
   int64_t chunk = total_tokens * n_kv_heads / want_blocks;
   const int round = step_tokens * kAttnUnroll;
   if (chunk < round) chunk = round;

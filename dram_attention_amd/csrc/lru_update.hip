@@ -21,11 +21,6 @@
 // Bound: latency; algorithmic bytes are the metadata only.
 #include "lru_keys.hpp"
 
-// Optional phase stamps for profiling builds (expands to nothing otherwise).
-#ifndef DA_LRU_STAMP
-#define DA_LRU_STAMP(n)
-#endif
-
 namespace da {
 
 constexpr int kLruMaxK = 8192;  // distinct-miss list kept in LDS (parallel path)
@@ -68,7 +63,6 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
   int32_t *mslot = miss_slot_out + (int64_t)h * K;
   int32_t *slot_epoch = slot_epoch_all ? slot_epoch_all + (int64_t)h * n_hbm : nullptr;
 
-  DA_LRU_STAMP(0);
   const int32_t step = *step_ptr + (bump ? 1 : 0);
   const TimeT now = (TimeT)step;
 
@@ -135,7 +129,6 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
     }
     if (t == 0) sm.n_miss = 0;
     __syncthreads();
-    DA_LRU_STAMP(1);
     // -- phase B: rank the first occurrences in visiting order ---------------
     for (int base = 0; base < K; base += kSelThreads) {
       const int k = base + t;
@@ -163,7 +156,6 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       __syncthreads();
     }
     const int m = (int)sm.n_miss;
-    DA_LRU_STAMP(2);
     // -- phase C: the m least recently used slots, in eviction order ---------
     const uint32_t *victims = nullptr;
     if (m > 0 && cand_all != nullptr && m <= k_cand) {
@@ -191,7 +183,6 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       LeastRecentKey<TimeT> key{time};
       victims = select_sorted(key, n_hbm, m, sm.sel);
     }
-    DA_LRU_STAMP(3);
     // -- phase D: hand slot i to the i-th distinct missed page ---------------
     for (int i = t; i < m; i += kSelThreads) {
       const int32_t p = sm.miss_page[i];
@@ -206,7 +197,6 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       if (slot_epoch) slot_epoch[v] = step;
     }
     if (t == 0) miss_count[h] = m;
-    DA_LRU_STAMP(4);
   }
 
   // The last head to finish publishes the bumped step and re-arms the ticket for
@@ -220,7 +210,6 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       *ticket = 0;
     }
   }
-  DA_LRU_STAMP(5);
 }
 
 // One 256-thread block per (entry, head), striding over the head's miss list.

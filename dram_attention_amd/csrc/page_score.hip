@@ -12,9 +12,6 @@
 // keeps its slice of up to kRows query rows in registers, accumulates in fp32
 // and the kLanes partial sums are folded with wavefront shuffles.
 #include "common.hpp"
-#ifdef DA_TUNE
-#include <stdlib.h>
-#endif
 
 namespace da {
 
@@ -166,17 +163,11 @@ static void launch_vec(const void *q, int64_t qrs, int64_t qhs, const void *mm, 
                        int n_heads, int64_t n_pages, OutT *out, int64_t ors, int64_t ohs,
                        int round_out, hipStream_t s) {
   constexpr int kGroups = 64 / kLanes;
-  // rounds per block: enough blocks to fill the part a few times over, but each
-  // block amortises its query load over several rounds of pages
-  int rounds = 1;
-#ifdef DA_TUNE
-  if (const char *e = getenv("DA_SCORE_ROUNDS")) rounds = atoi(e);
-#endif
+  // rounds of pages per block: one, i.e. as many blocks as the row allows (several
+  // rounds per block, amortising the query load, measured no faster)
+  const int rounds = 1;
   if (n_rows <= 4) {
-#ifndef DA_SCORE_UNROLL
-#define DA_SCORE_UNROLL 2
-#endif
-    constexpr int kRows = 4, kUnroll = DA_SCORE_UNROLL;
+    constexpr int kRows = 4, kUnroll = 2;
     dim3 grid((unsigned)ceil_div(n_pages, 4 * kGroups * kUnroll * rounds), n_heads, 1);
     hipLaunchKernelGGL((page_score_vec_kernel<T, kLanes, kRows, kUnroll, OutT>), grid, dim3(256),
                        0, s, (const char *)q, qrs, qhs, (const char *)mm, n_rows, n_pages, out,
