@@ -532,12 +532,16 @@ def test_graph_replay_equals_eager_steps(fused):
     assert same(graphed.cache_k[0, :c], eager.cache_k[0, :c])
 
 
-def test_static_prefix_equals_full_attention():
+@pytest.mark.parametrize("full_size", [False, True])
+def test_static_prefix_equals_full_attention(full_size):
     """Prefix within the HBM budget: the static cache path is dense attention over
-    the whole sequence (the 32K configuration through init_cache)."""
+    the whole sequence (the 32K configuration through init_cache, scaled down and
+    at its full size, configs[1])."""
     from dram_attention_amd import DRAMAttention, DummyCache
 
-    w = WORKLOADS["32k"].scaled(dram_tokens=4096, local_cache=512, lru_tokens=4096, steps=3)
+    w = WORKLOADS["32k"]
+    if not full_size:
+        w = w.scaled(dram_tokens=4096, local_cache=512, lru_tokens=4096, steps=3)
     prompt = make_prompt(w, 3)
     m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, 16, w.top_k_tokens, w.n_kv_heads,
                       w.head_dim, device=DEV, dtype=w.dtype)
@@ -545,7 +549,7 @@ def test_static_prefix_equals_full_attention():
     assert isinstance(m.lru_cache, DummyCache)
     inputs = DecodeInputs(w, prompt.q0, 3)
     ks, vs = [prompt.k[0]], [prompt.v[0]]
-    for t in range(w.steps):
+    for t in range(min(w.steps, 4)):
         xq, xk, xv = inputs.next()
         out = m(xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=w.prompt_tokens + t, stage="generate")
         ks.append(xk[0]); vs.append(xv[0])
@@ -555,12 +559,15 @@ def test_static_prefix_equals_full_attention():
 
 
 # ------------------------------------------------------------ full size, by properties
-def test_headline_size_invariants():
-    """configs[2] (128K prefix, 8192 pages/head) at full size: invariants that need
-    no CPU walk, plus attention against a dense fp32 computation on the GPU."""
+@pytest.mark.parametrize("name,steps", [("128k", 6), ("1m", 3)])
+def test_full_size_invariants(name, steps):
+    """configs[2] (128K prefix, 8192 pages/head) and configs[4] (1M prefix, 65536
+    pages/head, 64 query heads) at full size: invariants that need no CPU walk,
+    plus attention against a dense fp32 computation on the GPU."""
     from dram_attention_amd import DRAMAttention
 
-    w = WORKLOADS["128k"]
+    w = WORKLOADS[name]
+    H, rep, kp, D = w.n_kv_heads, w.rep, w.pages_per_q_head, w.head_dim
     prompt = make_prompt(w, 0)
     m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, 16, w.top_k_tokens, w.n_kv_heads,
                       w.head_dim, device=DEV, dtype=w.dtype)
@@ -570,27 +577,27 @@ def test_headline_size_invariants():
     inputs = DecodeInputs(w, prompt.q0, 0)
     N, P = w.n_hbm_pages, w.n_dram_pages
     ar = torch.arange(N, device=DEV)
-    for t in range(6):
+    for t in range(steps):
         xq, xk, xv = inputs.next()
         xq, xk, xv = xq.to(DEV), xk.to(DEV), xv.to(DEV)
         out = m(xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
         idx, d2h, h2d = lru._topk_idx, lru.dram_page_to_hbm_page_mapping, lru.hbm_page_to_dram_page_mapping
-        assert idx.shape == (8, 1024)
+        assert idx.shape == (H, rep * kp)
         # selection: sorted by (score desc, index asc) within each query head, and no
         # unselected page beats the last selected one
         scores = lru.top_k_selector._scores                         # (rep, H, P)
-        sel = idx.view(8, 4, 256)
-        s_sel = torch.gather(scores.transpose(0, 1), 2, sel)          # (H, rep, 256)
+        sel = idx.view(H, rep, kp)
+        s_sel = torch.gather(scores.transpose(0, 1), 2, sel)          # (H, rep, kp)
         assert torch.all((s_sel[..., :-1] > s_sel[..., 1:]) |
                          ((s_sel[..., :-1] == s_sel[..., 1:]) & (sel[..., :-1] < sel[..., 1:])))
-        mask = torch.ones(8, 4, P, dtype=torch.bool, device=DEV).scatter_(2, sel, False)
+        mask = torch.ones(H, rep, P, dtype=torch.bool, device=DEV).scatter_(2, sel, False)
         rest = scores.transpose(0, 1).masked_fill(~mask, -float("inf"))
         best_rest, best_idx = rest.max(dim=-1)
         last, last_idx = s_sel[..., -1], sel[..., -1]
         assert torch.all((best_rest < last) | ((best_rest == last) & (best_idx > last_idx)))
         # LRU maps: inverse of each other, all requests resident and touched now
-        assert same(torch.gather(d2h, 1, h2d), ar.expand(8, N))
-        assert (d2h >= 0).sum().item() == 8 * N
+        assert same(torch.gather(d2h, 1, h2d), ar.expand(H, N))
+        assert (d2h >= 0).sum().item() == H * N
         slots = torch.gather(d2h, 1, idx)
         assert torch.all(slots >= 0)
         assert torch.all(torch.gather(lru.page_access_time, 1, slots) == t + 1)
@@ -600,11 +607,11 @@ def test_headline_size_invariants():
         assert same(lru.hbm_kv_cache, want_pages)
         # attention over all resident slots ++ local window ++ new token
         c = w.prompt_tokens + t - w.dram_tokens
-        kk = torch.cat([lru.hbm_kv_cache.view(8, N * 16, 2, 128)[:, :, 0],
+        kk = torch.cat([lru.hbm_kv_cache.view(H, N * 16, 2, D)[:, :, 0],
                         m.cache_k[0, : c + 1].transpose(0, 1)], 1).float()
-        vv = torch.cat([lru.hbm_kv_cache.view(8, N * 16, 2, 128)[:, :, 1],
+        vv = torch.cat([lru.hbm_kv_cache.view(H, N * 16, 2, D)[:, :, 1],
                         m.cache_v[0, : c + 1].transpose(0, 1)], 1).float()
-        s = torch.einsum("hrd,htd->hrt", xq[0, 0].float().view(8, 4, 128), kk) / math.sqrt(128)
-        want = torch.einsum("hrt,htd->hrd", torch.softmax(s, -1), vv).reshape(32, 128)
+        s = torch.einsum("hrd,htd->hrt", xq[0, 0].float().view(H, rep, D), kk) / math.sqrt(D)
+        want = torch.einsum("hrt,htd->hrd", torch.softmax(s, -1), vv).reshape(H * rep, D)
         assert close(out[0, 0].float(), want, 2e-2, 1e-2)
         assert same(m.cache_k[0, c], xk[0, 0]) and same(m.cache_v[0, c], xv[0, 0])
