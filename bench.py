@@ -606,7 +606,7 @@ def main():
             "cache": type(layer.m.lru_cache).__name__,
         },
         "roofline": {
-            "bound": "hbm", "kernel": "decode_attention_split_kernel (prefix + local segments)",
+            "bound": "hbm", "kernel": "decode_attention_tile_kernel (first pass: prefix + local segments, matrix cores)",
             "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
             "algorithmic_bytes": attn_b, "avg_us": attn_us,

@@ -24,6 +24,9 @@
 // phase 2, issued once the page stream has finished, covers the re-assigned
 // slots through the miss list and then merges everything.  Both phases are the
 // same kernel; a chunk id says which segment a block works on.
+#include <type_traits>
+
+#include "attention_mfma.hpp"
 #include "page_stream.hpp"
 
 namespace da {
@@ -163,12 +166,31 @@ decode_attention_merge_kernel(const AttnArgs a, int mode, int head_dim, char *__
     lse_out[hq] = lt > 0.f ? (mx + __builtin_amdgcn_logf(lt)) * kLn2 : -INFINITY;
 }
 
+// The matrix-core form of the pass, for the shapes it takes.
+template <typename T, int kD>
+static void launch_tile(const AttnArgs &a, int n_launch, int n_kv_heads, hipStream_t s) {
+  const dim3 grid(n_launch, n_kv_heads, 1);
+  if (a.rep <= 4)
+    hipLaunchKernelGGL((decode_attention_tile_kernel<T, kD, 4>), grid, dim3(kAttnThreads), 0, s, a);
+  else if (a.rep <= 8)
+    hipLaunchKernelGGL((decode_attention_tile_kernel<T, kD, 8>), grid, dim3(kAttnThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((decode_attention_tile_kernel<T, kD, 16>), grid, dim3(kAttnThreads), 0, s, a);
+}
+
 template <typename T, int kLanes, bool kTail>
 static void launch_split(AttnArgs a, int first_chunk, int n_launch, int n_kv_heads,
                          hipStream_t s) {
   if (n_launch <= 0) return;
   a.chunk_base = first_chunk;
   const int rep = a.rep;
+  if constexpr (!kTail && T::kBytes == 2 && (kLanes == 8 || kLanes == 16 || kLanes == 32)) {
+    const int dtype = std::is_same<T, BF16>::value ? DA_BF16 : DA_F16;
+    if (tile_pass_supported(dtype, kLanes * 8, rep, a.slot_epoch != nullptr, a.page_size)) {
+      launch_tile<T, kLanes * 8>(a, n_launch, n_kv_heads, s);
+      return;
+    }
+  }
   // Up to 4 query rows per block; 8 (with a shorter unroll, ~240 vector registers,
   // two waves per SIMD) when the GQA group is that wide and rows are <= 256 bytes:
   // one read of K/V for 8 heads beats two reads for 4 + 4 (1M workload: 115 vs 137 us).

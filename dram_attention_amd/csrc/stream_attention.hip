@@ -3,6 +3,9 @@
 // grid (what da_decode_attention_paged issues for DA_PHASE_STREAM).  Neither
 // has a counterpart in the reference, which copies pages with index_select /
 // index_copy_ (dram_attention/lru_cache.py:224-241) before it attends.
+#include <type_traits>
+
+#include "attention_mfma.hpp"
 #include "page_stream.hpp"
 
 namespace da {
@@ -32,12 +35,38 @@ decode_stream_attend_kernel(const AttnArgs a, const GatherAttendArgs g, const in
   }
 }
 
+// The same with the matrix-core form of the attention pass (one block takes all
+// query rows of a kv head, so the grid has no row dimension).
+template <typename T, int kLanes, int kRowsAttn, int kRowsGather>
+__global__ void __launch_bounds__(kAttnThreads)
+decode_stream_attend_tile_kernel(const AttnArgs a, const GatherAttendArgs g, const int g_blocks) {
+  if ((int)blockIdx.x < g_blocks)
+    gather_attend_block<T, kLanes, kRowsGather>(g, blockIdx.y * g_blocks + blockIdx.x,
+                                                g_blocks * gridDim.y);
+  else
+    attention_tile_block<T, kLanes * 8, kRowsAttn>(a, (int)blockIdx.x - g_blocks);
+}
+
 // The page stream and the first attention pass as one launch.
 template <typename T, int kLanes>
 static void launch_stream_attend(AttnArgs a, const GatherAttendArgs &g, int g_blocks, int n_chunks,
                                  int n_kv_heads, hipStream_t s) {
   a.chunk_base = 0;
   const int rep = a.rep;
+  // (rows of 512 bytes stay with the vector pass here: both roles' LDS would not fit a block)
+  if constexpr (T::kBytes == 2 && (kLanes == 8 || kLanes == 16)) {
+    const int dtype = std::is_same<T, BF16>::value ? DA_BF16 : DA_F16;
+    if (tile_pass_supported(dtype, kLanes * 8, rep, a.slot_epoch != nullptr, a.page_size)) {
+      const dim3 grid(g_blocks + n_chunks, n_kv_heads, 1);
+      if (rep > 4)
+        hipLaunchKernelGGL((decode_stream_attend_tile_kernel<T, kLanes, 8, 8>), grid,
+                           dim3(kAttnThreads), 0, s, a, g, g_blocks);
+      else
+        hipLaunchKernelGGL((decode_stream_attend_tile_kernel<T, kLanes, 4, 4>), grid,
+                           dim3(kAttnThreads), 0, s, a, g, g_blocks);
+      return;
+    }
+  }
   if (rep > 4 && kLanes <= 16) {
     const dim3 grid(g_blocks + n_chunks, n_kv_heads, 1);
     hipLaunchKernelGGL((decode_stream_attend_kernel<T, (kLanes <= 16 ? kLanes : 16), 8, 8>), grid,
