@@ -577,7 +577,7 @@ def main():
     # HBM bytes per launch of the roofline kernel from the committed counter runs
     # (profiles/bench_128k_hbm_traffic_pmc.md: FETCH_SIZE x 2.0 + WRITE_SIZE); only
     # known for the workload those runs used
-    traffic = 152.5e6 if w.name == "128k" else None
+    traffic = 152.8e6 if w.name == "128k" else None
     result = {
         "metric": "decode steps/sec per layer at 128K ctx; scorer+attn HBM GB/s vs peak",
         "value": args.steps * n_layers / dt,
