@@ -95,6 +95,27 @@ decode_attention_merge_kernel(const AttnArgs a, int mode, int head_dim, char *__
     return tail_chunk0 + (i - n_first);
   };
 
+  // Partial rows: a thread owns four adjacent channels (one 16-byte lane) of every
+  // lanes_c-th live chunk, four rows in flight.  Their addresses do not depend on
+  // the statistics, so the first batch (usually all of them) is requested before
+  // the statistics are staged and reduced: one memory round trip instead of two.
+  __shared__ float sm_acc[kMergeThreads * 4];
+  const int quads = head_dim / 4;              // 16-byte lanes per row (head_dim % 4 == 0 here)
+  const int lanes_c = kMergeThreads / quads;   // chunk lanes
+  const int qd = t % quads, cl = t / quads;
+  const bool rows_mine = cl < lanes_c && cl < n_live;
+  float4 v[4];
+  auto load_rows = [&](int i0) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * lanes_c;
+      const int ic = i < n_live ? i : cl;  // clamp the address; the weight will be zero
+      const int64_t slot = (int64_t)chunk_of(ic) * a.n_q_heads + hq;
+      v[u] = *(const float4 *)(a.part_acc + slot * head_dim + qd * 4);
+    }
+  };
+  if (rows_mine) load_rows(cl);
+
   // Stage the (max, sum) pairs of the live chunks in LDS with one load per
   // thread, then let every wave reduce them for itself (no second barrier).
   __shared__ float2 sm_ml[kMergeStats];
@@ -121,30 +142,18 @@ decode_attention_merge_kernel(const AttnArgs a, int mode, int head_dim, char *__
   for (int d = 32; d >= 1; d >>= 1) lt += __shfl_xor(lt, d, 64);
   const float inv = lt > 0.f ? 1.f / lt : 0.f;
 
-  __shared__ float sm_acc[kMergeThreads * 4];
-  const int quads = head_dim / 4;              // 16-byte lanes per row (head_dim % 4 == 0 here)
-  const int lanes_c = kMergeThreads / quads;   // chunk lanes
-  const int qd = t % quads, cl = t / quads;
   float at[4] = {0.f, 0.f, 0.f, 0.f};
-  if (cl < lanes_c) {
-    // four independent partial rows in flight per thread
+  if (rows_mine) {
     for (int i0 = cl; i0 < n_live; i0 += 4 * lanes_c) {
-      float4 v[4];
-      float w[4];
+      if (i0 != cl) load_rows(i0);
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int i = i0 + u * lanes_c;
-        const int ic = i < n_live ? i : cl;  // clamp the address, zero the weight
-        const int64_t slot = (int64_t)chunk_of(ic) * a.n_q_heads + hq;
-        v[u] = *(const float4 *)(a.part_acc + slot * head_dim + qd * 4);
-        w[u] = i < n_live ? fast_exp2(stat(ic).x - mx) : 0.f;
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        at[0] = fmaf(v[u].x, w[u], at[0]);
-        at[1] = fmaf(v[u].y, w[u], at[1]);
-        at[2] = fmaf(v[u].z, w[u], at[2]);
-        at[3] = fmaf(v[u].w, w[u], at[3]);
+        const float w = i < n_live ? fast_exp2(stat(i).x - mx) : 0.f;
+        at[0] = fmaf(v[u].x, w, at[0]);
+        at[1] = fmaf(v[u].y, w, at[1]);
+        at[2] = fmaf(v[u].z, w, at[2]);
+        at[3] = fmaf(v[u].w, w, at[3]);
       }
     }
   }
