@@ -231,8 +231,11 @@ int da_pages_gather(const void *dram, int64_t dram_head_stride_bytes,
  *   new_k, new_v : (Hkv, D) of the current token (head stride new_head_stride),
  *                  or NULL to attend over the c_len cached rows only
  *   out          : (Hq, D) in `dtype`;  lse_out : optional (Hq) fp32, natural log
- * fp32 accumulation throughout; 16-bit query/key products use packed dot
- * instructions.
+ * fp32 accumulation throughout.  bf16/fp16 inputs with head_dim 64, 128 or 256
+ * and at most 16 query heads per kv head run both products on the matrix
+ * cores (the softmax weights are rounded to the input type for the second
+ * product, as flash-attn rounds them); other shapes use packed dot
+ * instructions on the vector units.
  * workspace: da_decode_attention_workspace_bytes(...) bytes, 16-byte aligned, no
  * initial state; `miss_tokens` is 0 here (see da_decode_attention_paged).
  */
