@@ -162,22 +162,28 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       // The caller's list of the k_cand least recent slots, made before this call
       // touched anything: untouched slots keep their order and still precede every
       // touched one, so the first m untouched entries are the victims.
-      const int32_t slot = t < k_cand ? cand_all[(int64_t)h * k_cand + t] : 0;
-      const bool untouched = t < k_cand && time[slot] != now;
-      const uint64_t m_un = __ballot(untouched);
-      if (lane == 0) sm.wave_count[wave] = (uint32_t)__popcll(m_un);
-      __syncthreads();
-      uint32_t before = 0, total = 0;
+      uint32_t kept = 0;  // untouched entries found so far (the same in every thread)
+      for (int base = 0; base < k_cand && kept < (uint32_t)m; base += kSelThreads) {
+        const int i = base + t;
+        const int32_t slot = i < k_cand ? cand_all[(int64_t)h * k_cand + i] : 0;
+        const bool untouched = i < k_cand && time[slot] != now;
+        const uint64_t m_un = __ballot(untouched);
+        if (lane == 0) sm.wave_count[wave] = (uint32_t)__popcll(m_un);
+        __syncthreads();
+        uint32_t before = 0, total = 0;
 #pragma unroll
-      for (int w = 0; w < kSelWaves; ++w) {
-        const uint32_t c = sm.wave_count[w];
-        if (w < wave) before += c;
-        total += c;
+        for (int w = 0; w < kSelWaves; ++w) {
+          const uint32_t c = sm.wave_count[w];
+          if (w < wave) before += c;
+          total += c;
+        }
+        const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+        if (untouched)
+          sm.sel.idx_out[kept + before + (uint32_t)__popcll(m_un & below)] = (uint32_t)slot;
+        kept += total;
+        __syncthreads();  // idx_out is complete so far; wave_count may be rewritten
       }
-      const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-      if (untouched) sm.sel.idx_out[before + (uint32_t)__popcll(m_un & below)] = (uint32_t)slot;
-      __syncthreads();
-      if (total >= (uint32_t)m) victims = sm.sel.idx_out;  // else: too many were touched
+      if (kept >= (uint32_t)m) victims = sm.sel.idx_out;  // else: too many were touched
     }
     if (m > 0 && victims == nullptr) {
       LeastRecentKey<TimeT> key{time};
@@ -275,8 +281,8 @@ extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_i
                              const int32_t *candidates, int k_cand, void *workspace,
                              size_t workspace_bytes, void *stream) {
   using namespace da;
-  DA_REQUIRE(k_cand >= 0 && k_cand <= kSelThreads && (k_cand == 0 || candidates != nullptr),
-             "da_lru_update: bad candidate list (%d entries, at most %d)", k_cand, kSelThreads);
+  DA_REQUIRE(k_cand >= 0 && k_cand <= kSelMaxK && (k_cand == 0 || candidates != nullptr),
+             "da_lru_update: bad candidate list (%d entries, at most %d)", k_cand, kSelMaxK);
   DA_REQUIRE(n_kv_heads >= 0 && k >= 0 && n_dram_pages >= 0 && n_hbm_pages >= 0,
              "da_lru_update: bad geometry (heads %d k %d pages %lld slots %d)", n_kv_heads, k,
              (long long)n_dram_pages, n_hbm_pages);

@@ -91,9 +91,9 @@ extern "C" int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_
              out_itype);
   LruCandidateArgs cand = {};
   if (candidates != nullptr && k_cand > 0) {
-    DA_REQUIRE(access_time && n_hbm_pages > 0 && k_cand <= n_hbm_pages && k_cand <= kSelThreads,
+    DA_REQUIRE(access_time && n_hbm_pages > 0 && k_cand <= n_hbm_pages && k_cand <= kSelMaxK,
                "da_topk_pages_lru: %d candidates of %d slots (at most %d)", k_cand, n_hbm_pages,
-               kSelThreads);
+               kSelMaxK);
     DA_REQUIRE(time_type == DA_TIME_F32 || time_type == DA_TIME_I32,
                "da_topk_pages_lru: bad access-time type");
     cand.access_time = access_time;

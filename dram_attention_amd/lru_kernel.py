@@ -36,12 +36,26 @@ class LruScratch(NamedTuple):
             miss_count=torch.zeros(num_heads, dtype=torch.int32, device=device),
             hit_mask=torch.empty(num_heads, max(k, 1), dtype=torch.uint8, device=device),
             workspace=torch.zeros(ws, dtype=torch.uint8, device=device),
-            candidates=torch.empty(num_heads, max(min(num_hbm_pages, MAX_LRU_CANDIDATES), 1),
+            candidates=torch.empty(num_heads, max(lru_candidate_count(k, num_hbm_pages), 1),
                                    dtype=torch.int32, device=device),
         )
 
 
-MAX_LRU_CANDIDATES = 256  # least recent slots listed ahead of an update (one sort block's fast path)
+MIN_LRU_CANDIDATES = 256   # one sort block's fast path
+MAX_LRU_CANDIDATES = 8192  # what one workgroup orders in LDS
+
+
+def lru_candidate_count(k: int, num_hbm_pages: int) -> int:
+    """Least recent slots to list ahead of an update with ``k`` requests per head.  Up
+    to 1024 requests: what the sort's short path handles, so that the list does not
+    lengthen the top-k launch; it covers the misses of a typical step there (an eighth
+    of the requests at the 128K workload), and a step that misses more falls back to
+    ordering all slots inside the update.  Beyond that (the 1M workload: as many
+    requests as slots, two thirds of the slots touched and a third replaced in every
+    step) only the complete order is sure to hold enough untouched slots, and the
+    longer top-k launch hides its cost."""
+    want = MIN_LRU_CANDIDATES if k <= 1024 else num_hbm_pages
+    return min(num_hbm_pages, MAX_LRU_CANDIDATES, want)
 
 
 def lru_update(

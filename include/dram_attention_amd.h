@@ -135,7 +135,7 @@ int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
  * da_lru_update that follows (see its `candidates`).  The order of the slots
  * does not depend on this step's scores, so it is computed next to the top-k
  * instead of inside the LRU update, which every later launch of the step waits
- * for.  Needs n_heads == Hkv; k_cand <= min(N_hbm, 1024); candidates == NULL or
+ * for.  Needs n_heads == Hkv; k_cand <= min(N_hbm, 8192); candidates == NULL or
  * k_cand == 0 gives plain da_topk_pages.  n_rows == 0 or kp == 0 with a list
  * requested computes the list only.
  */

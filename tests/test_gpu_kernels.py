@@ -302,10 +302,12 @@ def test_lru_update_matches_serial_walk(H, P, N, K, itype, ttype, pinned):
 
 
 @pytest.mark.parametrize("H,P,N,K,ttype", [
-    (8, 8192, 2048, 1024, torch.float32),     # the 128K layer: list of 512, ~120 victims per step
+    (8, 8192, 2048, 1024, torch.float32),     # the 128K layer: list of 256, ~120 victims per step
     (4, 1024, 256, 200, torch.float32),       # list of 256 with up to 200 of them touched: falls back
-    (2, 4096, 600, 64, torch.int32),          # list of 512 of 600 slots
+    (2, 4096, 600, 64, torch.int32),          # list of 256 of 600 slots
     (3, 300, 100, 37, torch.float32),
+    (2, 16384, 4096, 4096, torch.float32),    # the 1M layer's shape: list of 2048, filtered in two rounds
+    (2, 9000, 3000, 2500, torch.int32),       # list of 1250: a partial second round
 ])
 def test_lru_update_with_candidate_list_matches_serial_walk(H, P, N, K, ttype):
     """Victims taken from the list of least recent slots made ahead of the update
