@@ -26,11 +26,6 @@
 
 #include "common.hpp"
 
-// Optional phase stamps for profiling builds (expands to nothing otherwise).
-#ifndef DA_SEL_STAMP
-#define DA_SEL_STAMP(n)
-#endif
-
 namespace da {
 
 constexpr int kSelThreads = 1024;
@@ -113,7 +108,6 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     }
   };
 
-  DA_SEL_STAMP(8);
   uint32_t low_or = 0, low_and = 0xffffu;
   for (int s = n_seg - 1; s >= 0; --s) {  // ends with segment 0 in registers
     load_segment(s);
@@ -131,7 +125,6 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     low_or |= __shfl_xor(low_or, d, 64);
     low_and &= __shfl_xor(low_and, d, 64);
   }
-  DA_SEL_STAMP(0);
   for (int i = t; i < 256 * kHistCopies; i += kSelThreads) sm.hist[i] = 0;
   if (t < kSelRankSortMax) sm.rank[t] = 0;
   if (t == 0) {
@@ -145,7 +138,6 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     atomicAnd(&sm.low_and, low_and & 0xffffu);
   }
 
-  DA_SEL_STAMP(1);
   uint32_t prefix = 0;  // the digits of T fixed so far (high bits)
   int passes = 4;
   for (int pass = 0; pass < passes; ++pass) {
@@ -205,7 +197,6 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     __syncthreads();
     prefix = (prefix << 8) | sm.digit;
   }
-  DA_SEL_STAMP(2);
   const bool low_const = passes == 2;
   const uint32_t thresh = low_const ? (prefix << 16) | sm.low_or : prefix;  // k-th largest key
   const uint32_t n_eq = sm.remaining;                                       // keys == T to keep
@@ -253,7 +244,6 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     }
     __syncthreads();
   }
-  DA_SEL_STAMP(3);
 
   if (k <= kSelRankSortMax) {
     // Rank counting: thread (e, slice) counts the words of its slice that beat
@@ -284,7 +274,6 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     __syncthreads();
     if (slice == 0 && e < k) sm.idx_out[sm.rank[e]] = 0xffffffffu - (uint32_t)mine;
     __syncthreads();
-    DA_SEL_STAMP(4);
     return sm.idx_out;
   }
 
