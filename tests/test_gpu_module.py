@@ -280,6 +280,16 @@ def test_decode_parity_cpu_reference_config():
     assert 0.0 < rate < 1.0
 
 
+@pytest.mark.parametrize("name,steps", [("128k", 64), ("1m", 8)])
+def test_decode_parity_full_size(name, steps):
+    """configs[2] for all of its 64 steps and configs[4] for its first 8, at full size,
+    step by step against the oracle (which is fed the kernel's scores): request lists,
+    hit masks, both maps, access times and slot payload bit for bit, attention within
+    the bf16 tolerance; the position stays on the device."""
+    rate = run_parity(WORKLOADS[name], 0, steps, atol=2e-2, rtol=1e-2, device_pos=True)
+    assert 0.5 < rate < 0.95
+
+
 def test_decode_parity_bf16_scaled_llama_shape():
     """The 128K layer shape scaled to a prefix the oracle walks in seconds."""
     w = WORKLOADS["128k"].scaled(dram_tokens=16384, local_cache=1024, lru_tokens=4096,
