@@ -578,6 +578,7 @@ def main():
     # (profiles/bench_128k_hbm_traffic_pmc.md: FETCH_SIZE x 2.0 + WRITE_SIZE); only
     # known for the workload those runs used
     traffic = 152.8e6 if w.name == "128k" else None
+    paged = isinstance(layer.m.lru_cache, LRUCache)
     result = {
         "metric": "decode steps/sec per layer at 128K ctx; scorer+attn HBM GB/s vs peak",
         "value": args.steps * n_layers / dt,
@@ -606,7 +607,12 @@ def main():
             "cache": type(layer.m.lru_cache).__name__,
         },
         "roofline": {
-            "bound": "hbm", "kernel": "decode_attention_tile_kernel (first pass: prefix + local segments, matrix cores)",
+            "bound": "hbm",
+            "kernel": ("decode_attention_tile_kernel (first pass: prefix + local segments, matrix cores)"
+                       if paged else
+                       "decode_attention_tile_kernel + merge launch (static prefix: the two launches "
+                       "of one call are timed together, so frac is a lower bound for the first)")
+                      if w.dtype != torch.float32 else "decode_attention_split_kernel (fp32, vector units)",
             "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
             "algorithmic_bytes": attn_b, "avg_us": attn_us,
