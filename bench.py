@@ -95,7 +95,6 @@ class Layer:
             self.m._workspace = None
         inputs = DecodeInputs(w, prompt.q0, seed)
         qs, ks, vs = zip(*(inputs.next() for _ in range(total_steps)))
-        self.host_inputs = (qs, ks, vs)
         self.qs = torch.cat(qs).to(dev)   # (T, 1, Hq, D)
         self.ks = torch.cat(ks).to(dev)
         self.vs = torch.cat(vs).to(dev)
@@ -260,31 +259,63 @@ def host_link_gbps(dev, mb=64, reps=5):
     return reps * (mb << 20) / (time.perf_counter() - t0) / 1e9
 
 
-def cpu_baseline(w, layer, steps):
-    """The CPU oracle (a restatement of the reference's torch/Triton path) on the
-    first `steps` decode steps of the same workload, all host cores."""
-    from oracle import dram_attention_oracle as O
-
-    o = O.DecodeOracle(steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
-                       w.n_kv_heads, w.head_dim, dtype=w.dtype)
-    o.init_cache(layer.prompt.k, layer.prompt.v)
-    qs, ks, vs = layer.host_inputs
-    cpu_model = "unknown"
+def cpu_model_name():
     try:
         with open("/proc/cpuinfo") as f:
-            cpu_model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")),
-                             cpu_model)
+            return next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")),
+                        "unknown")
     except OSError:
-        pass
+        return "unknown"
+
+
+def time_oracle(w, seed, steps, warmup=0, prompt=None):
+    """Wall-clock of the CPU oracle on `warmup` untimed + `steps` timed decode steps
+    of workload `w`.  Draws its own prompt and step inputs from the workload's
+    seeded generators (the first steps the GPU run sees), so it depends on
+    nothing the GPU legs staged.  Returns (steps/s, per-stage ms per step)."""
+    from dram_attention_amd.synthetic import DecodeInputs, make_prompt
+    from oracle import dram_attention_oracle as O
+
+    if prompt is None:
+        prompt = make_prompt(w, seed)
+    o = O.DecodeOracle(warmup + steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                       w.n_kv_heads, w.head_dim, dtype=w.dtype)
+    o.init_cache(prompt.k, prompt.v)
+    inputs = DecodeInputs(w, prompt.q0, seed)
+    for t in range(warmup):
+        o.generate(*inputs.next(), w.prompt_tokens + t)
     stages = {}
+    staged = [inputs.next() for _ in range(steps)]
     t0 = time.perf_counter()
-    for t in range(steps):
-        o.generate(qs[t], ks[t], vs[t], w.prompt_tokens + t, timings=stages)
+    for t, (q, k, v) in enumerate(staged):
+        o.generate(q, k, v, w.prompt_tokens + warmup + t, timings=stages)
     dt = time.perf_counter() - t0
-    return {"value": steps / dt, "unit": "decode steps/s per layer", "cores": torch.get_num_threads(),
-            "kind": "port", "cpu_model": cpu_model, "stage_ms_per_step": {k: v / steps * 1e3 for k, v in stages.items()},
-            "sample": f"first {steps} decode steps of workload {w.name}, torch-CPU oracle, "
-                      f"{dt / steps * 1e3:.1f} ms/step"}
+    return steps / dt, {k: v / steps * 1e3 for k, v in stages.items()}, dt
+
+
+def cpu_baseline(w, seed, steps, prompt=None, cfg0_steps=16, cfg0_warmup=3):
+    """The CPU oracle (a restatement of the reference's torch/Triton path; the
+    reference has no CPU path of its own for the LRU walk or for attention) on
+    all host cores: `value` on the first `steps` decode steps of the benchmarked
+    workload, `cfg0` on configs[0] exactly as stated (fp32, 3 warm-up + 16 timed)."""
+    from dram_attention_amd.synthetic import WORKLOADS
+
+    cores = torch.get_num_threads()
+    value, stages, dt = time_oracle(w, seed, steps, prompt=prompt)
+    res = {"value": value, "unit": "decode steps/s per layer", "cores": cores, "kind": "port",
+           "cpu_model": cpu_model_name(), "os_cpu_count": os.cpu_count(),
+           "same_workload": True, "stage_ms_per_step": stages,
+           "sample": f"first {steps} decode steps of workload {w.name}, torch-CPU oracle, "
+                     f"{dt / steps * 1e3:.1f} ms/step, {dt:.1f} s in all"}
+    if cfg0_steps > 0:
+        w0 = WORKLOADS["cpu"]
+        v0, st0, dt0 = time_oracle(w0, seed, cfg0_steps, warmup=cfg0_warmup)
+        res["cfg0"] = {"value": v0, "unit": "decode steps/s per layer", "cores": cores,
+                       "stage_ms_per_step": st0,
+                       "sample": f"configs[0] as stated: fp32, 8q/2kv heads, D 64, 8192-token prefix, "
+                                 f"{cfg0_warmup} warm-up + {cfg0_steps} timed steps, "
+                                 f"{dt0 / cfg0_steps * 1e3:.2f} ms/step"}
+    return res
 
 
 def time_cache_build(layer, dev):
@@ -637,10 +668,11 @@ def main():
                 result[name] = value
         except Exception as exc:  # noqa: BLE001 - reported, not swallowed
             result[name] = {"error": f"{type(exc).__name__}: {exc}"}
+            print(f"bench.py: leg {name} failed: {type(exc).__name__}: {exc}", file=sys.stderr, flush=True)
 
     leg("cache_build", lambda: time_cache_build(layer, dev))
     if args.cpu_steps > 0:
-        leg("cpu_baseline", lambda: cpu_baseline(w, layer, args.cpu_steps))
+        leg("cpu_baseline", lambda: cpu_baseline(w, args.seed, args.cpu_steps, prompt=layer.prompt))
     if args.reference_shaped_steps > 3 and isinstance(layer.m.lru_cache, LRUCache):
         del layer, layers, model_step
         torch.cuda.empty_cache()

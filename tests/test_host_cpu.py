@@ -152,3 +152,20 @@ def test_layer_cache_file_round_trip(tmp_path):
     torch.save({"cache_k": k}, layer_cache_path(str(tmp_path), 9))
     with pytest.raises(KeyError):
         load_layer_cache(str(tmp_path), 9, device="cpu")
+
+
+def test_bench_cpu_baseline_is_independent_of_staged_steps():
+    """The CPU-baseline leg of bench.py draws its own inputs: it must work for any
+    --steps/--warmup of the GPU legs (the driver runs --steps 20 --warmup 5 with the
+    default 64 oracle steps) and must report value, cores and the CPU model."""
+    import bench
+    from dram_attention_amd.synthetic import WORKLOADS
+
+    w = WORKLOADS["128k"].scaled(name="128k/32", dram_tokens=4096, local_cache=256,
+                                 lru_tokens=1024, top_k_tokens=256)
+    res = bench.cpu_baseline(w, seed=0, steps=64, cfg0_steps=2, cfg0_warmup=1)
+    assert res["value"] > 0 and res["cores"] >= 1 and res["kind"] == "port"
+    assert res["cpu_model"] and "error" not in res
+    assert "64 decode steps" in res["sample"]
+    assert res["cfg0"]["value"] > 0
+    assert set(res["stage_ms_per_step"]) == {"score", "top_k", "lru", "attention"}
