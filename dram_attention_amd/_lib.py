@@ -72,6 +72,13 @@ SIGNATURES = {
          c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
          c_void_p, c_int64, c_float, c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p],
     ),
+    "da_decode_attention_static_capacity": (c_size_t, []),
+    "da_decode_attention_static": (
+        c_int,
+        [c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_int64,
+         c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+         c_void_p, c_int64, c_float, c_void_p, c_int64, c_void_p, c_void_p],
+    ),
     "da_decode_attention_paged": (
         c_int,
         [c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_int64,

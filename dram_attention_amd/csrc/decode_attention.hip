@@ -465,3 +465,76 @@ extern "C" int da_decode_attention(const void *q, int64_t q_head_stride, int n_q
                                    new_head_stride, scale, out, out_head_stride, lse_out,
                                    workspace, workspace_bytes, nullptr, stream);
 }
+
+// ---- the same attention for callers that cannot allocate -------------------
+// The partial results live in a file-scope device array instead of a workspace
+// the caller brings.  The array's name is only a host-side handle: the device
+// address is looked up once per device with hipGetSymbolAddress and kept; every
+// GPU holds its own copy of the array at its own address.
+namespace da {
+constexpr size_t kStaticScratchBytes = DA_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void *volatile scratch_ptr[kMaxDevices];  // device address of `scratch`, per device
+
+// Device address of `scratch` on the current device.  Two threads that race on
+// the first call both look the address up and store the same value.
+static int static_scratch(void **ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return fail((int)e, "da_decode_attention_static: hipGetDevice: %s", hipGetErrorString(e));
+  }
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(DA_ENOTSUP, "da_decode_attention_static: device %d beyond the %d this library tracks",
+                dev, kMaxDevices);
+  void *p = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return fail(e != hipSuccess ? (int)e : DA_EINVAL,
+                  "da_decode_attention_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    }
+    __atomic_store_n(&scratch_ptr[dev], p, __ATOMIC_RELEASE);
+  }
+  *ptr = p;
+  return DA_OK;
+}
+}  // namespace da
+
+extern "C" size_t da_decode_attention_static_capacity(void) { return da::kStaticScratchBytes; }
+
+extern "C" int da_decode_attention_static(const void *q, int64_t q_head_stride, int n_q_heads,
+                                          int n_kv_heads, int head_dim, int dtype, const void *pk,
+                                          const void *pv, int64_t p_tok_stride,
+                                          int64_t p_head_stride, int64_t p_len, void *ck, void *cv,
+                                          int64_t c_tok_stride, int64_t c_head_stride,
+                                          int64_t c_capacity, int64_t c_len,
+                                          const int32_t *c_len_dev, const void *new_k,
+                                          const void *new_v, int64_t new_head_stride, float scale,
+                                          void *out, int64_t out_head_stride, float *lse_out,
+                                          void *stream) {
+  using namespace da;
+  const size_t need = da_decode_attention_workspace_bytes(n_q_heads, n_kv_heads, head_dim, dtype,
+                                                          p_len, c_capacity, 0);
+  if (need == 0)
+    return fail(DA_EINVAL, "da_decode_attention_static: bad shape (heads %d/%d, head_dim %d, dtype %d, "
+                "lengths %lld/%lld)", n_q_heads, n_kv_heads, head_dim, dtype, (long long)p_len,
+                (long long)c_capacity);
+  if (need > kStaticScratchBytes)
+    return fail(DA_ENOTSUP,
+                "da_decode_attention_static: this shape needs %zu bytes of partial results, the "
+                "built-in buffer holds %zu; use da_decode_attention with a workspace",
+                need, kStaticScratchBytes);
+  void *ws = nullptr;
+  int rc = static_scratch(&ws);
+  if (rc) return rc;
+  return da_decode_attention_paged(q, q_head_stride, n_q_heads, n_kv_heads, head_dim, dtype, pk, pv,
+                                   p_tok_stride, p_head_stride, p_len, ck, cv, c_tok_stride,
+                                   c_head_stride, c_capacity, c_len, c_len_dev, new_k, new_v,
+                                   new_head_stride, scale, out, out_head_stride, lse_out, ws,
+                                   kStaticScratchBytes, nullptr, stream);
+}

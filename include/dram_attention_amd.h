@@ -253,6 +253,32 @@ int da_decode_attention(const void *q, int64_t q_head_stride, int n_q_heads,
                         size_t workspace_bytes, void *stream);
 
 /*
+ * da_decode_attention for callers that cannot allocate device memory or bring a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference.  Same arguments
+ * and results as da_decode_attention, minus the workspace: the partial results
+ * of the split pass live in a device array built into the library,
+ * DA_STATIC_SCRATCH_BYTES per GPU for the life of the process
+ * (da_decode_attention_static_capacity() returns the figure).  The call makes
+ * no hipMalloc / hipFree.  Shapes whose partial results exceed the array
+ * (da_decode_attention_workspace_bytes(..., miss_tokens = 0) > capacity) are
+ * refused with DA_ENOTSUP and nothing is launched.  All calls on one GPU share
+ * that GPU's array: calls that overlap in time on one GPU (two streams, two
+ * threads) race; calls that follow each other on one stream do not, and no
+ * state is carried from one call to the next.
+ */
+#define DA_STATIC_SCRATCH_BYTES (8u << 20)
+size_t da_decode_attention_static_capacity(void);
+int da_decode_attention_static(const void *q, int64_t q_head_stride, int n_q_heads,
+                               int n_kv_heads, int head_dim, int dtype, const void *pk,
+                               const void *pv, int64_t p_tok_stride, int64_t p_head_stride,
+                               int64_t p_len, void *ck, void *cv, int64_t c_tok_stride,
+                               int64_t c_head_stride, int64_t c_capacity, int64_t c_len,
+                               const int32_t *c_len_dev, const void *new_k, const void *new_v,
+                               int64_t new_head_stride, float scale, void *out,
+                               int64_t out_head_stride, float *lse_out, void *stream);
+
+/*
  * The same attention when the prefix is the slot array of the LRU page cache
  * and the missed pages of this step are streamed in concurrently on another
  * stream (no counterpart in the reference, whose page copies and attention are
