@@ -43,6 +43,44 @@ def _hipcc() -> str:
     return exe
 
 
+def check_hand_placed_registers(verbose: bool = False) -> None:
+    """The tile scorer (csrc/page_score_tile.hpp) places a few vector instructions by
+    inline asm, which the compiler's tracking of matrix-core hazards does not see.
+    Its safety rule is that those instructions write only registers no MFMA of the
+    kernel ever names as an operand or destination.  This reads the compiler's own
+    listing of page_score.hip and fails the build if any variant breaks the rule."""
+    import re
+
+    hipcc = _hipcc()
+    listing = HERE / "build" / "page_score.s"
+    cmd = [hipcc, *[f for f in HIPCC_FLAGS if f != "-fPIC"], "-S", "--cuda-device-only",
+           str(CSRC / "page_score.hip"), "-o", str(listing)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc -S failed on page_score.hip:\n{proc.stderr}")
+    text = listing.read_text()
+    names = re.findall(r"^(_ZN2da22page_score_tile_kernel[^\s:]*):", text, re.M)
+    if not names:
+        raise RuntimeError("no page_score_tile_kernel in the listing of page_score.hip")
+    for name in names:
+        start = text.index("\n" + name + ":")
+        body = text[start:text.index("s_endpgm", start)]
+        placed = {int(r) for _, r in re.findall(
+            r"^\s+(v_dot2_f32_bf16|v_bfi_b32|v_mov_b32) v(\d+),", body, re.M)}
+        matrix = set()
+        for operands in re.findall(r"v_mfma\S+ (.*)", body):
+            for lo, hi in re.findall(r"v\[(\d+):(\d+)\]", operands):
+                matrix.update(range(int(lo), int(hi) + 1))
+        if len(placed) != 12 or not matrix:
+            raise RuntimeError(f"{name}: expected 12 hand-placed destinations and some MFMAs, "
+                               f"found {len(placed)} and {len(matrix)} registers")
+        if placed & matrix:
+            raise RuntimeError(f"{name}: registers {sorted(placed & matrix)} are written by "
+                               "hand-placed instructions and used by an MFMA")
+    if verbose:
+        print(f"hand-placed registers of {len(names)} tile scorer variants are clear of MFMA operands")
+
+
 def build_library(verbose: bool = False) -> Path:
     """Compile every kernel source and link the shared library; returns its path."""
     hipcc = _hipcc()
@@ -68,6 +106,7 @@ def build_library(verbose: bool = False) -> Path:
     proc = subprocess.run(link, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stderr}")
+    check_hand_placed_registers(verbose)
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
 

@@ -11,7 +11,10 @@
 // scores 64/kLanes pages per step from fully used cache lines.  Each lane
 // keeps its slice of up to kRows query rows in registers, accumulates in fp32
 // and the kLanes partial sums are folded with wavefront shuffles.
+#include <type_traits>
+
 #include "common.hpp"
+#include "page_score_tile.hpp"
 
 namespace da {
 
@@ -186,13 +189,34 @@ template <typename T, typename OutT>
 static int launch_page_score(const void *q, int64_t qrs, int64_t qhs, const void *mm,
                              int64_t mhs, int64_t mps, int64_t mrs, int n_rows, int n_heads,
                              int64_t n_pages, int head_dim, OutT *out, int64_t ors, int64_t ohs,
-                             int round_out, hipStream_t s) {
+                             int round_out, bool ordered, hipStream_t s) {
   constexpr int V = T::kVec;
   const int lanes = head_dim % V == 0 ? head_dim / V : 0;
   const bool vec = lanes >= 1 && lanes <= 64 && is_pow2(lanes) && mrs == head_dim &&
                    mps == 2 * (int64_t)head_dim && mhs == n_pages * 2 * head_dim &&
                    qrs % V == 0 && qhs % V == 0 && ((uintptr_t)q % 16) == 0 &&
                    ((uintptr_t)mm % 16) == 0 && n_heads <= 65535 && n_rows <= 8 * 65535;
+  if constexpr (std::is_same<T, BF16>::value && std::is_same<OutT, float>::value) {
+    // bf16 summaries with ordered bounds, fp32 scores: the decode step's form
+    if (vec && ordered && n_rows <= 8 * 65535 &&
+        page_score_tile_supported(head_dim, n_pages, ors, ohs, out, q, mm, qrs, qhs)) {
+      const bool wide = n_rows > 4;
+      switch (head_dim) {
+        case 32:
+          if (wide) launch_page_score_tile<1, 8>(q, qrs, qhs, mm, n_rows, n_heads, n_pages, out, ors, ohs, round_out, s);
+          else launch_page_score_tile<1, 4>(q, qrs, qhs, mm, n_rows, n_heads, n_pages, out, ors, ohs, round_out, s);
+          break;
+        case 64:
+          if (wide) launch_page_score_tile<2, 8>(q, qrs, qhs, mm, n_rows, n_heads, n_pages, out, ors, ohs, round_out, s);
+          else launch_page_score_tile<2, 4>(q, qrs, qhs, mm, n_rows, n_heads, n_pages, out, ors, ohs, round_out, s);
+          break;
+        default:
+          if (wide) launch_page_score_tile<4, 8>(q, qrs, qhs, mm, n_rows, n_heads, n_pages, out, ors, ohs, round_out, s);
+          else launch_page_score_tile<4, 4>(q, qrs, qhs, mm, n_rows, n_heads, n_pages, out, ors, ohs, round_out, s);
+      }
+      return launch_status("da_page_score");
+    }
+  }
   if (vec) {
 #define DA_SCORE_CASE(L)                                                                     \
   case L:                                                                                    \
@@ -231,13 +255,13 @@ template <typename T>
 static int dispatch_out(const void *q, int64_t qrs, int64_t qhs, const void *mm, int64_t mhs,
                         int64_t mps, int64_t mrs, int n_rows, int n_heads, int64_t n_pages,
                         int head_dim, void *out, int64_t ors, int64_t ohs, bool out_f32,
-                        int round_out, hipStream_t s) {
+                        int round_out, bool ordered, hipStream_t s) {
   if (out_f32)
     return launch_page_score<T, float>(q, qrs, qhs, mm, mhs, mps, mrs, n_rows, n_heads, n_pages,
-                                       head_dim, (float *)out, ors, ohs, round_out, s);
+                                       head_dim, (float *)out, ors, ohs, round_out, ordered, s);
   typedef typename Storage<T>::type O;
   return launch_page_score<T, O>(q, qrs, qhs, mm, mhs, mps, mrs, n_rows, n_heads, n_pages,
-                                 head_dim, (O *)out, ors, ohs, round_out, s);
+                                 head_dim, (O *)out, ors, ohs, round_out, ordered, s);
 }
 
 }  // namespace da
@@ -246,8 +270,7 @@ extern "C" int da_page_score(const void *q, int64_t q_row_stride, int64_t q_head
                              const void *minmax, int64_t mm_head_stride, int64_t mm_page_stride,
                              int64_t mm_r_stride, int n_rows, int n_heads, int64_t n_pages,
                              int head_dim, int dtype, void *out, int64_t out_row_stride,
-                             int64_t out_head_stride, int out_dtype, int round_to_input,
-                             void *stream) {
+                             int64_t out_head_stride, int out_dtype, int flags, void *stream) {
   using namespace da;
   DA_REQUIRE(n_rows >= 0 && n_heads >= 0 && n_pages >= 0 && head_dim > 0,
              "da_page_score: bad geometry (rows %d heads %d pages %lld dim %d)", n_rows, n_heads,
@@ -258,20 +281,24 @@ extern "C" int da_page_score(const void *q, int64_t q_row_stride, int64_t q_head
              "da_page_score: out_dtype must be fp32 or the input dtype");
   if (n_rows == 0 || n_heads == 0 || n_pages == 0) return DA_OK;
   DA_REQUIRE(q && minmax && out, "da_page_score: null pointer");
+  DA_REQUIRE((flags & ~(DA_SCORE_ROUND | DA_SCORE_ORDERED_BOUNDS)) == 0,
+             "da_page_score: unknown flag bits %d", flags);
   hipStream_t s = (hipStream_t)stream;
   const bool out_f32 = out_dtype == DA_F32;
+  const int round_to_input = flags & DA_SCORE_ROUND;
+  const bool ordered = (flags & DA_SCORE_ORDERED_BOUNDS) != 0;
   switch (dtype) {
     case DA_F32:
       return dispatch_out<F32>(q, q_row_stride, q_head_stride, minmax, mm_head_stride,
                                mm_page_stride, mm_r_stride, n_rows, n_heads, n_pages, head_dim,
-                               out, out_row_stride, out_head_stride, true, 0, s);
+                               out, out_row_stride, out_head_stride, true, 0, ordered, s);
     case DA_F16:
       return dispatch_out<F16>(q, q_row_stride, q_head_stride, minmax, mm_head_stride,
                                mm_page_stride, mm_r_stride, n_rows, n_heads, n_pages, head_dim,
-                               out, out_row_stride, out_head_stride, out_f32, round_to_input, s);
+                               out, out_row_stride, out_head_stride, out_f32, round_to_input, ordered, s);
     default:
       return dispatch_out<BF16>(q, q_row_stride, q_head_stride, minmax, mm_head_stride,
                                 mm_page_stride, mm_r_stride, n_rows, n_heads, n_pages, head_dim,
-                                out, out_row_stride, out_head_stride, out_f32, round_to_input, s);
+                                out, out_row_stride, out_head_stride, out_f32, round_to_input, ordered, s);
   }
 }

@@ -13,9 +13,15 @@ import torch
 from . import _lib
 
 
+DA_SCORE_ROUND, DA_SCORE_ORDERED_BOUNDS = 1, 2
+
+
 def page_scores(q: torch.Tensor, min_max: torch.Tensor, out: torch.Tensor,
-                round_to_input: bool) -> torch.Tensor:
-    """score[n,h,l] into ``out`` (fp32 or q.dtype; any strides, last axis dense)."""
+                round_to_input: bool, ordered_bounds: bool = False) -> torch.Tensor:
+    """score[n,h,l] into ``out`` (fp32 or q.dtype; any strides, last axis dense).
+    ``ordered_bounds``: the caller vouches that min_max[...,0,:] <= min_max[...,1,:]
+    (summaries made by page_min_max are); the kernel may then pick the bound by the
+    sign of q instead of forming both products."""
     N, H, D = q.shape
     H1, L, R, D1 = min_max.shape
     assert H1 == H and D1 == D and R == 2
@@ -35,7 +41,9 @@ def page_scores(q: torch.Tensor, min_max: torch.Tensor, out: torch.Tensor,
             min_max.data_ptr(), min_max.stride(0), min_max.stride(1), min_max.stride(2),
             N, H, L, D, _lib.dtype_code(q.dtype),
             out.data_ptr(), out.stride(0), out.stride(1), _lib.dtype_code(out.dtype),
-            int(round_to_input), _lib.stream_ptr(q.device),
+            (DA_SCORE_ROUND if round_to_input else 0)
+            | (DA_SCORE_ORDERED_BOUNDS if ordered_bounds else 0),
+            _lib.stream_ptr(q.device),
         ),
         "da_page_score",
     )

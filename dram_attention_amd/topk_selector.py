@@ -101,7 +101,9 @@ class IPUpperboundTopKSelector:
             qv = q[0, 0].view(H, rep, head_dim).transpose(0, 1)
         else:
             qv = q[0].view(seq_len, H, rep, head_dim).transpose(1, 2).reshape(n_rows, H, head_dim)
-        return page_scores(qv, self.chunk_min_max, self._scores, round_to_input=True)
+        # chunk_min_max comes from page_min_max: min <= max in every channel
+        return page_scores(qv, self.chunk_min_max, self._scores, round_to_input=True,
+                           ordered_bounds=True)
 
     def top_k(self, q: torch.Tensor, k: int) -> torch.Tensor:
         """Indices of the top k pages, (seq_len, num_kv_heads, rep, k) int64, best first."""

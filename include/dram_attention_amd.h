@@ -98,17 +98,28 @@ int da_pages_build(const void *k, const void *v, int64_t tok_stride, int64_t hea
  *   out    : (n_rows, H, L) with element strides (out_row_stride, out_head_stride, 1);
  *            out_dtype is DA_F32 or equal to `dtype`.
  * Arithmetic follows the reference kernel: for 16-bit inputs each product is
- * rounded to the input type, the maximum and the sum over D are fp32; when
- * `round_to_input` is non-zero the fp32 sum is rounded to the input type
- * before it is stored (the value the reference ranks on, :99), also when
- * out_dtype is DA_F32.
+ * rounded to the input type, the maximum and the sum over D are fp32.  `flags`:
+ *   DA_SCORE_ROUND          : the fp32 sum is rounded to the input type before it
+ *                             is stored (the value the reference ranks on, :99),
+ *                             also when out_dtype is DA_F32
+ *   DA_SCORE_ORDERED_BOUNDS : the caller vouches that minmax[h,l,0,d] <=
+ *                             minmax[h,l,1,d] everywhere (or both NaN), as
+ *                             da_page_minmax writes them.  The larger product is
+ *                             then q * (q >= 0 ? max : min): same values, and
+ *                             bf16 summaries with fp32 output and head_dim 32,
+ *                             64 or 128 take a kernel with less than half the
+ *                             vector instructions (products by packed dot
+ *                             instructions, the sum over D on the matrix cores).
+ *                             With bounds that are not ordered the result is
+ *                             the sum of those products, not the reference's.
  */
+#define DA_SCORE_ROUND 1
+#define DA_SCORE_ORDERED_BOUNDS 2
 int da_page_score(const void *q, int64_t q_row_stride, int64_t q_head_stride,
                   const void *minmax, int64_t mm_head_stride, int64_t mm_page_stride,
                   int64_t mm_r_stride, int n_rows, int n_heads, int64_t n_pages,
                   int head_dim, int dtype, void *out, int64_t out_row_stride,
-                  int64_t out_head_stride, int out_dtype, int round_to_input,
-                  void *stream);
+                  int64_t out_head_stride, int out_dtype, int flags, void *stream);
 
 /*
  * Subsystem 3 — ordered top-k page selection per score row.

@@ -73,7 +73,10 @@ def max_ip(q: torch.Tensor, min_max: torch.Tensor) -> torch.Tensor:
         qn = q[n].reshape(H, 1, D)
         lo = (qn * min_max[:, :, 0, :])  # rounded to dt by torch for 16-bit types
         hi = (qn * min_max[:, :, 1, :])
-        best = torch.maximum(lo.float(), hi.float())
+        # tl.maximum with its default PropagateNan.NONE (:80): a NaN product loses
+        # against the other one, as with fmax; max_ip_ref's amax (:132) would
+        # propagate it, the two statements differ only there
+        best = torch.fmax(lo.float(), hi.float())
         out[n] = best.sum(dim=-1, dtype=torch.float32).to(dt)
     return out
 

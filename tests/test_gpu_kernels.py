@@ -107,6 +107,99 @@ def test_page_score_strided_query_view():
     assert same(out.cpu(), out.cpu().bfloat16().float())
 
 
+def ordered_summaries(H, L, D, seed):
+    """Random (H, L, 2, D) bf16 summaries with min <= max in every channel."""
+    a = torch.randn(H, L, 2, D, generator=gen(seed)).bfloat16()
+    return torch.stack((torch.minimum(a[:, :, 0], a[:, :, 1]), torch.maximum(a[:, :, 0], a[:, :, 1])), dim=2)
+
+
+def check_scores(got, want, changed_frac=0.02):
+    """Same rounding points as the oracle; the fp32 summation order differs, so a sum
+    on a bf16 rounding boundary may land on the neighbouring value: one step, rarely."""
+    got, want = got.float().cpu(), want.float()
+    diff = (got - want).abs()
+    assert torch.all(diff <= want.abs() * 2.0 ** -7 + 1e-30)
+    assert (diff > 0).float().mean().item() < changed_frac
+
+
+@pytest.mark.parametrize("N,H,D,L", [
+    (4, 8, 128, 8192),      # the decode shape of the 128K workload: one round of 8 steps
+    (8, 8, 128, 3000),      # 8 query rows, ragged page count
+    (4, 2, 128, 70001),     # several rounds per wave, odd length
+    (8, 3, 128, 40000),     # 8 rows, several rounds
+    (4, 8, 64, 2048), (8, 2, 64, 777), (4, 4, 32, 515), (8, 1, 32, 4096),
+    (1, 1, 128, 1), (3, 2, 128, 5), (5, 2, 128, 33), (12, 2, 128, 130), (4, 8, 128, 2048),
+])
+def test_page_score_ordered_bounds_matches_oracle(N, H, D, L):
+    """The decode step's scorer (bf16 summaries with min <= max, fp32 output): bound picked
+    by the sign of q, products by packed dot instructions, sum over D on the matrix cores."""
+    from dram_attention_amd.max_ip_kernel import page_scores
+
+    q = torch.randn(N, H, D, generator=gen(N * 1000 + L)).bfloat16()
+    mm = ordered_summaries(H, L, D, seed=L + D)
+    for rounded in (True, False):
+        out = torch.full((N, H, L), float("nan"), dtype=torch.float32, device=DEV)
+        page_scores(q.to(DEV), mm.to(DEV), out, round_to_input=rounded, ordered_bounds=True)
+        if rounded:
+            check_scores(out, O.max_ip(q, mm))
+            assert same(out.cpu(), out.cpu().bfloat16().float())
+        else:
+            # unrounded sums: against the plain kernel (both products, max, vector sum)
+            plain = torch.empty_like(out)
+            page_scores(q.to(DEV), mm.to(DEV), plain, round_to_input=False, ordered_bounds=False)
+            terms = (q.float()[:, :, None, None, :] * mm.float()[None]).abs().amax(dim=3).sum(-1)
+            assert torch.all((out - plain).abs().cpu() <= 1e-6 * terms + 1e-30)
+
+
+def test_page_score_ordered_bounds_special_values():
+    """Signed zeros and denormal-range products in the query, and non-finite bounds: a
+    page with an infinite or NaN bound scores as the reference kernel's formula says
+    (+-inf, NaN, or, where a zero query channel meets an infinite bound, the other
+    product: tl.maximum drops a NaN operand), and leaves its neighbours alone."""
+    from dram_attention_amd.max_ip_kernel import page_scores
+
+    N, H, D, L = 4, 2, 128, 200
+    q = torch.randn(N, H, D, generator=gen(70)).bfloat16()
+    q[0, 0, :8] = 0.0
+    q[1, 0, :8] = -0.0
+    q[2, 1, 5] = 1e-30
+    mm = ordered_summaries(H, L, D, seed=71)
+    inf = float("inf")
+    mm[0, 3, 1, 7] = inf                       # max = +inf
+    mm[0, 4, 0, 9] = -inf                      # min = -inf
+    mm[1, 5, :, 11] = float("nan")             # NaN in both bounds (what aminmax gives)
+    mm[1, 6, 0, 2], mm[1, 6, 1, 2] = -inf, inf
+    mm[1, 7, :, 0] = 1e-38                     # tiny bounds
+    out = torch.empty(N, H, L, dtype=torch.float32, device=DEV)
+    page_scores(q.to(DEV), mm.to(DEV), out, round_to_input=True, ordered_bounds=True)
+    want = O.max_ip(q, mm).float()
+    got = out.cpu()
+    special = torch.zeros(H, L, dtype=torch.bool)
+    for h, l in ((0, 3), (0, 4), (1, 5), (1, 6)):
+        special[h, l] = True
+    assert same(got[:, special], want[:, special])          # inf / NaN exactly as the formula
+    assert not torch.isfinite(want[:, special]).all()
+    assert torch.isfinite(want[:2, 0, 3]).all()             # zero query channel x infinite bound
+    # the plain kernel (both products, fmax) agrees entry for entry on where they are finite
+    plain = torch.empty_like(out)
+    page_scores(q.to(DEV), mm.to(DEV), plain, round_to_input=True, ordered_bounds=False)
+    assert same(torch.isfinite(plain.cpu()), torch.isfinite(got))
+    assert same(torch.isnan(plain.cpu()), torch.isnan(got))
+    check_scores(got[:, ~special], want[:, ~special])
+
+
+def test_page_score_ordered_bounds_strided_query_view():
+    from dram_attention_amd.max_ip_kernel import page_scores
+
+    for Hkv, rep, D, L in ((8, 4, 128, 8192), (8, 8, 128, 4100), (2, 4, 64, 300)):
+        q = torch.randn(1, 1, Hkv * rep, D, generator=gen(21 + rep)).bfloat16()
+        mm = ordered_summaries(Hkv, L, D, seed=22)
+        qv = q.to(DEV)[0, 0].view(Hkv, rep, D).transpose(0, 1)
+        out = torch.empty(rep, Hkv, L, dtype=torch.float32, device=DEV)
+        page_scores(qv, mm.to(DEV), out, round_to_input=True, ordered_bounds=True)
+        check_scores(out, O.scores_for_selection(q, mm))
+
+
 # ------------------------------------------------------------------ top-k
 def run_topk(scores, rep, k):
     from dram_attention_amd.topk_selector import topk_pages

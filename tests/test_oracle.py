@@ -68,6 +68,32 @@ def test_max_ip_quest_statement():
     assert torch.allclose(O.max_ip(q, mm), (q[:, :, None, :] * pick).sum(-1), atol=1e-5)
 
 
+def test_max_ip_nan_product_loses_against_the_other_product():
+    """tl.maximum with its default (PropagateNan.NONE, the reference kernel's call at
+    max_ip_triton_kernel.py:80) returns the other operand when one product is NaN:
+    0 * inf contributes max(0 * min, NaN) = 0 * min, not NaN.  Both NaN stays NaN."""
+    q = torch.tensor([[[0.0, 2.0]]])                                   # (1, 1, 2)
+    mm = torch.tensor([[[[1.0, -1.0], [float("inf"), 3.0]]]])          # min (1,-1), max (inf,3)
+    assert O.max_ip(q, mm).item() == 0.0 * 1.0 + 2.0 * 3.0
+    mm_nan = torch.tensor([[[[float("nan"), -1.0], [float("nan"), 3.0]]]])
+    assert torch.isnan(O.max_ip(torch.tensor([[[1.0, 2.0]]]), mm_nan)).all()
+    # hand-written loop over the same rule
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(2, 1, 6, generator=g)
+    q[0, 0, 2] = 0.0
+    mm = torch.randn(1, 3, 2, 6, generator=g)
+    mm[0, 1, 1, 2] = float("inf")
+    want = torch.zeros(2, 1, 3)
+    for n in range(2):
+        for l in range(3):
+            acc = 0.0
+            for d in range(6):
+                a, b = float(q[n, 0, d] * mm[0, l, 0, d]), float(q[n, 0, d] * mm[0, l, 1, d])
+                acc += b if a != a else (a if b != b else max(a, b))
+            want[n, 0, l] = acc
+    assert torch.allclose(O.max_ip(q, mm), want, atol=1e-5)
+
+
 def test_max_ip_bf16_rounding_points():
     g = torch.Generator().manual_seed(6)
     q = torch.randn(2, 2, 32, generator=g).bfloat16()
