@@ -55,6 +55,9 @@ def parse_args():
     ap.add_argument("--force-lru", action="store_true",
                     help="workload 32k: run the page-cache path although the prefix fits the cache "
                          "(every request hits; the reference's init_cache would pick the static cache)")
+    ap.add_argument("--plain-scorer", action="store_true",
+                    help="score pages with the plain vector kernel (both products and their maximum) "
+                         "instead of the sign-select / matrix-core form: same scores, for comparison")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-steps", type=int, default=64, help="steps of the CPU oracle to time (0 = skip)")
     ap.add_argument("--reference-shaped-steps", type=int, default=24,
@@ -532,6 +535,8 @@ def main():
     for li in range(max(args.layers, 1)):
         layers.append(Layer(w, args.seed + li, total, dev, overlap=not args.no_overlap,
                             force_lru=args.force_lru))
+        if args.plain_scorer and isinstance(layers[-1].m.lru_cache, LRUCache):
+            layers[-1].m.lru_cache.top_k_selector.bounds_are_ordered = False
         if li > 0:
             layers[-1].prompt = None   # only layer 0 feeds the CPU baseline
         if args.layers > 1:
@@ -636,6 +641,7 @@ def main():
             "page_stream": "serialised" if args.no_overlap else "in the launch of the first attention pass",
             "seed": args.seed,
             "cache": type(layer.m.lru_cache).__name__,
+            "scorer": "plain vector kernel" if args.plain_scorer else "sign-select + matrix-core sum",
         },
         "roofline": {
             "bound": "hbm",

@@ -64,19 +64,38 @@ def check_hand_placed_registers(verbose: bool = False) -> None:
         raise RuntimeError("no page_score_tile_kernel in the listing of page_score.hip")
     for name in names:
         start = text.index("\n" + name + ":")
-        body = text[start:text.index("s_endpgm", start)]
-        placed = {int(r) for _, r in re.findall(
-            r"^\s+(v_dot2_f32_bf16|v_bfi_b32|v_mov_b32) v(\d+),", body, re.M)}
-        matrix = set()
-        for operands in re.findall(r"v_mfma\S+ (.*)", body):
-            for lo, hi in re.findall(r"v\[(\d+):(\d+)\]", operands):
-                matrix.update(range(int(lo), int(hi) + 1))
+        lines = text[start:text.index("s_endpgm", start)].splitlines()
+        placed, matrix, labels, loops = {}, {}, {}, []
+        for n, line in enumerate(lines):
+            m = re.match(r"\s+(v_dot2_f32_bf16|v_bfi_b32|v_mov_b32) v(\d+),", line)
+            if m:
+                placed.setdefault(int(m.group(2)), []).append(n)
+            m = re.match(r"\s+v_mfma\S+ (.*)", line)
+            if m:
+                for lo, hi in re.findall(r"v\[(\d+):(\d+)\]", m.group(1)):
+                    for r in range(int(lo), int(hi) + 1):
+                        matrix.setdefault(r, []).append(n)
+            m = re.match(r"(\.LBB\w+):", line)
+            if m:
+                labels[m.group(1)] = n
+            m = re.match(r"\s+s_cbranch\w*\s+(\.LBB\w+)|\s+s_branch\s+(\.LBB\w+)", line)
+            if m:
+                target = labels.get(m.group(1) or m.group(2))
+                if target is not None:          # a label already seen: a backward branch, i.e. a loop
+                    loops.append((target, n))
         if len(placed) != 12 or not matrix:
             raise RuntimeError(f"{name}: expected 12 hand-placed destinations and some MFMAs, "
                                f"found {len(placed)} and {len(matrix)} registers")
-        if placed & matrix:
-            raise RuntimeError(f"{name}: registers {sorted(placed & matrix)} are written by "
-                               "hand-placed instructions and used by an MFMA")
+        # A register may serve both only when every MFMA that names it comes after
+        # the last hand-placed write to it (the variable behind it is dead by then),
+        # in straight-line code: never inside a loop that also holds such a write.
+        for r in sorted(set(placed) & set(matrix)):
+            last_write, first_use = max(placed[r]), min(matrix[r])
+            in_one_loop = any(lo <= w <= hi and lo <= u <= hi for lo, hi in loops
+                              for w in placed[r] for u in matrix[r])
+            if first_use < last_write or in_one_loop:
+                raise RuntimeError(f"{name}: register v{r} is written by a hand-placed "
+                                   "instruction while an MFMA may still use it")
     if verbose:
         print(f"hand-placed registers of {len(names)} tile scorer variants are clear of MFMA operands")
 

@@ -134,22 +134,30 @@ page_score_tile_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t
                  : "=v"(t_sel[e]), "=v"(t_lo[e]), "=v"(t_hi[e]));
   }
 
-  // query operands of this lane's 8 channels: (q, 0) and (0, q) words for the
-  // two products of a pair, and the sign mask that picks max (q >= 0) or min
-  uint32_t qlo[kRows][4], qhi[kRows][4], pick[kRows][4];
+  // the query words of this lane's 8 channels, requested first and unpacked only
+  // after the first round's page loads have gone out (loads complete in order)
+  u32x4 qw[kRows];
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
     const int n = row0 + r < n_rows ? row0 + r : n_rows - 1;
-    const u32x4 w = load16(q + (n * q_row_stride + h * q_head_stride + (int64_t)chunk * 8) * 2);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const uint32_t word = w[e];
-      qlo[r][e] = word & 0x0000ffffu;
-      qhi[r][e] = word & 0xffff0000u;
-      // each half: all ones when its sign bit is clear (packed arithmetic shift, then not)
-      pick[r][e] = ~__builtin_bit_cast(uint32_t, __builtin_bit_cast(score_i16x2, word) >> 15);
-    }
+    qw[r] = load16(q + (n * q_row_stride + h * q_head_stride + (int64_t)chunk * 8) * 2);
   }
+  // query operands: (q, 0) and (0, q) words for the two products of a pair, and
+  // the sign mask that picks max (q >= 0) or min
+  uint32_t qlo[kRows][4], qhi[kRows][4], pick[kRows][4];
+  auto unpack_query = [&]() {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t word = qw[r][e];
+        qlo[r][e] = word & 0x0000ffffu;
+        qhi[r][e] = word & 0xffff0000u;
+        // each half: all ones when its sign bit is clear (packed arithmetic shift, then not)
+        pick[r][e] = ~__builtin_bit_cast(uint32_t, __builtin_bit_cast(score_i16x2, word) >> 15);
+      }
+    }
+  };
   // indicator operands: column c of the product, as B, receives the row sums
   score_bf16x8 route[kRpa * 4];
 #pragma unroll
@@ -165,13 +173,15 @@ page_score_tile_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t
   // page of (round, step, row) and the loads of a round (addresses clamped
   // into the head: scores of pages beyond the end are not stored)
   auto first_page = [&](int round) { return ((int64_t)round * n_waves + wave_id) * kWavePages; };
+  const uint32_t last_page = (uint32_t)(n_pages - 1);   // page ids fit 31 bits (checked by the launcher)
+  const char *lane_base = head_base + chunk * 16;
   auto issue = [&](int round, u32x4 *vmin, u32x4 *vmax) {
-    const int64_t base = first_page(round) + (int64_t)pi * kSteps;
+    const int64_t first = first_page(round) + (int64_t)pi * kSteps;
+    const uint32_t base = first < n_pages ? (uint32_t)first : last_page;
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
-      int64_t p = base + s;
-      if (p >= n_pages) p = n_pages - 1;
-      const char *src = head_base + p * 2 * kRowBytes + chunk * 16;
+      const uint32_t p = base + s < last_page ? base + s : last_page;
+      const char *src = lane_base + (uint64_t)p * (2 * kRowBytes);
       vmin[s] = load16(src);
       vmax[s] = load16(src + kRowBytes);
     }
@@ -227,11 +237,15 @@ page_score_tile_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t
     if (first_page(0) >= n_pages) return;
     u32x4 vmin[kSteps], vmax[kSteps];
     issue(0, vmin, vmax);
+    __builtin_amdgcn_sched_barrier(0);   // all of the round's loads go out before anything waits
+    unpack_query();
     compute(0, vmin, vmax);
   } else {
     // two register sets: the next round's loads are in flight while this one is scored
     u32x4 amin[kSteps], amax[kSteps], bmin[kSteps], bmax[kSteps];
     issue(0, amin, amax);
+    __builtin_amdgcn_sched_barrier(0);
+    unpack_query();
     for (int round = 0; round < rounds; round += 2) {
       issue(round + 1, bmin, bmax);   // clamped: harmless when there is no such round
       compute(round, amin, amax);
@@ -246,6 +260,7 @@ inline bool page_score_tile_supported(int head_dim, int64_t n_pages, int64_t out
                                       int64_t out_head_stride, const void *out, const void *q,
                                       const void *mm, int64_t q_row_stride, int64_t q_head_stride) {
   return (head_dim == 32 || head_dim == 64 || head_dim == 128) && n_pages >= 1 &&
+         n_pages < ((int64_t)1 << 31) - 64 &&
          (uintptr_t)q % 16 == 0 && (uintptr_t)mm % 16 == 0 && q_row_stride % 8 == 0 &&
          q_head_stride % 8 == 0;
 }

@@ -81,6 +81,10 @@ class IPUpperboundTopKSelector:
         self.device = torch.device(device)
         # the summaries are built on the GPU: host-resident keys are moved first
         self.chunk_min_max = page_min_max(k_cache.to(device=device), num_pages)
+        # chunk_min_max comes from page_min_max, so min <= max in every channel and the
+        # scorer may pick the bound by the sign of q; clear this after writing other
+        # contents into chunk_min_max
+        self.bounds_are_ordered = True
         self._scores = None
 
     def scores(self, q: torch.Tensor) -> torch.Tensor:
@@ -101,9 +105,8 @@ class IPUpperboundTopKSelector:
             qv = q[0, 0].view(H, rep, head_dim).transpose(0, 1)
         else:
             qv = q[0].view(seq_len, H, rep, head_dim).transpose(1, 2).reshape(n_rows, H, head_dim)
-        # chunk_min_max comes from page_min_max: min <= max in every channel
         return page_scores(qv, self.chunk_min_max, self._scores, round_to_input=True,
-                           ordered_bounds=True)
+                           ordered_bounds=self.bounds_are_ordered)
 
     def top_k(self, q: torch.Tensor, k: int) -> torch.Tensor:
         """Indices of the top k pages, (seq_len, num_kv_heads, rep, k) int64, best first."""
