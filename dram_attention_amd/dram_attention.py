@@ -275,6 +275,26 @@ class DRAMAttention(torch.nn.Module):
         over resident pages, local window and the new token (appended in place).
         The missed pages stream in on a side stream while attention already
         covers the local window and every slot that keeps its page."""
+        return self.attend_(xq, xk, xv, start_pos, self.select_(xq))
+
+    def select_(self, xq: torch.Tensor):
+        """First half of a decode step: page scores, ordered top-k and the LRU update
+        (three launches that touch neither the host link nor K/V).  Returns what
+        :meth:`attend_` needs to finish the step, or None with a static cache.  The
+        two halves may be issued on different streams as long as attend_ is ordered
+        after select_ of the same step and before select_ of the next one."""
+        bsz, seqlen, Hq, D = xq.shape
+        if seqlen != 1:
+            raise RuntimeError("generate handles one token per call")
+        lru = self.lru_cache
+        if not isinstance(lru, LRUCache):
+            return None
+        idx = lru.select_(xq)
+        return idx, lru.update_(idx)
+
+    def attend_(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, start_pos, selected):
+        """Second half of a decode step: the page stream for the misses select_ found
+        and attention over resident pages, local window and the new token."""
         bsz, seqlen, Hq, D = xq.shape
         if seqlen != 1:
             raise RuntimeError("generate handles one token per call")
@@ -297,8 +317,7 @@ class DRAMAttention(torch.nn.Module):
                              out=out[0, 0], cache_len_offset=offset)
             return out
 
-        idx = lru.select_(xq)
-        scratch = lru.update_(idx)
+        idx, scratch = selected
         prefix_k, prefix_v = lru.views()
         if self._workspace is None:
             self._workspace = attention_workspace(

@@ -280,8 +280,11 @@ class DecodeOracle:
         self.dram_kv_cache_size = None
         self.uses_lru = False
 
-    def init_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor):
-        """k_cache, v_cache: (1, S, Hkv, D)."""
+    def init_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor, force_lru: bool = False):
+        """k_cache, v_cache: (1, S, Hkv, D).  `force_lru` builds the page cache even when
+        the prefix fits it (what constructing LRUCache directly over the prefix gives,
+        lru_cache.py:188-190 only asks for num_hbm_pages <= num_dram_pages): every page
+        is resident from the start and every request hits."""
         bsz, S, H, D = k_cache.shape
         assert bsz == 1, "Only support batch size 1"
         self.dram_kv_cache_size = dram_split(S, self.local_cache_size, self.page_size)
@@ -290,7 +293,7 @@ class DecodeOracle:
         self.cache_v[:tail] = v_cache[0, self.dram_kv_cache_size:]
         pk = k_cache[0, : self.dram_kv_cache_size].transpose(0, 1).contiguous()
         pv = v_cache[0, : self.dram_kv_cache_size].transpose(0, 1).contiguous()
-        self.uses_lru = self.dram_kv_cache_size > self.lru_hbm_cache_size
+        self.uses_lru = force_lru or self.dram_kv_cache_size > self.lru_hbm_cache_size
         if self.uses_lru:
             P = self.dram_kv_cache_size // self.page_size
             n_hbm = self.lru_hbm_cache_size // self.page_size

@@ -11,6 +11,7 @@ import torch
 from dram_attention_amd.synthetic import WORKLOADS, DecodeInputs, make_prompt
 from oracle import dram_attention_oracle as O
 
+from tests.parity import check_step
 from tests.util import close, same
 
 pytestmark = pytest.mark.gpu
@@ -139,8 +140,9 @@ def test_module_init_and_errors():
 
 
 def test_init_cache_from_layer_file(tmp_path):
-    """A layer set up from the chat example's cache file decodes like one set up from
-    the tensors themselves."""
+    """A layer set up from the chat example's cache file holds the page store the oracle
+    packs from the same K/V, decodes step by step like the oracle, and like a layer
+    set up from the tensors themselves."""
     from dram_attention_amd import DRAMAttention, save_layer_cache
 
     w = WORKLOADS["128k"].scaled(dram_tokens=4096, local_cache=256, lru_tokens=1024,
@@ -157,12 +159,20 @@ def test_init_cache_from_layer_file(tmp_path):
             m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
         mods.append(m)
     assert same(mods[0].lru_cache.dram_kv_cache, mods[1].lru_cache.dram_kv_cache)
+    # the page store built from the file is the reference's layout of the file's K/V
+    S = mods[0].dram_kv_cache_size
+    assert same(mods[0].lru_cache.dram_kv_cache,
+                O.pack_pages(prompt.k[0, :S].transpose(0, 1), prompt.v[0, :S].transpose(0, 1), w.page_size))
+    o = O.DecodeOracle(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                       w.n_kv_heads, w.head_dim, dtype=w.dtype)
+    o.init_cache(prompt.k, prompt.v)
     inputs = DecodeInputs(w, prompt.q0, 11)
     for t in range(w.steps):
-        xq, xk, xv = (x.to(DEV) for x in inputs.next())
-        a = mods[0](xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
-        b = mods[1](xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
+        xq, xk, xv = inputs.next()
+        a = mods[0](xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=w.prompt_tokens + t, stage="generate")
+        b = mods[1](xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=w.prompt_tokens + t, stage="generate")
         assert same(a, b)
+        check_step(mods[0], o, xq, xk, xv, w.prompt_tokens + t, a, t, 2e-2, 1e-2)
 
 
 def test_module_prefill_then_generate_shapes():
@@ -250,21 +260,10 @@ def run_parity(w, seed, steps, atol, rtol, device_pos=False):
         out = m(xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=pos if device_pos else start,
                 stage="generate")
         pos += 1
-        scores = lru.top_k_selector._scores.cpu()
-        own = O.scores_for_selection(xq, o.min_max)
-        assert torch.all((scores - own).abs() <= own.abs() * 2.0 ** -7 + 1e-4), f"scores, step {t}"
-        want = o.generate(xq, xk, xv, start, scores=scores)
-        assert same(lru._topk_idx.cpu(), o.last_idx), f"selection, step {t}"
+        check_step(m, o, xq, xk, xv, start, out, t, atol, rtol)
         if t == 0:
             for h, page in prompt.planted:
                 assert (o.last_idx[h] == page).any(), "planted page not selected"
-        assert lru.current_step.item() == o.state.step == t + 1
-        assert np.array_equal(lru.page_access_time.cpu().numpy(), o.state.time), f"time, step {t}"
-        assert np.array_equal(lru.dram_page_to_hbm_page_mapping.cpu().numpy(), o.state.d2h)
-        assert np.array_equal(lru.hbm_page_to_dram_page_mapping.cpu().numpy(), o.state.h2d)
-        assert np.array_equal(lru._scratch.hit_mask.cpu().numpy().astype(bool), o.last_hit)
-        assert same(lru.hbm_kv_cache.cpu(), o.hbm), f"slot payload, step {t}"
-        assert close(out.cpu().float(), want.float(), atol, rtol), f"output, step {t}"
         hits += int(o.last_hit.sum())
         total += o.last_hit.size
     c = w.prompt_tokens + steps - w.dram_tokens
@@ -489,7 +488,8 @@ def test_attention_on_the_page_stream_equals_tail_pass(base, kw):
 def test_graph_replay_equals_eager_steps(fused):
     """The whole step (selection, LRU, page stream on its side stream, two-phase
     attention, append) captured once and replayed: every replay, with eager work
-    and synchronisations in between, gives the eager module's bits and state."""
+    and synchronisations in between, matches the CPU oracle step by step (state bit
+    for bit, output within tolerance) and gives the eager module's bits and state."""
     from dram_attention_amd import DRAMAttention
 
     w = WORKLOADS["128k"].scaled(dram_tokens=16384, local_cache=1024, lru_tokens=4096,
@@ -503,8 +503,12 @@ def test_graph_replay_equals_eager_steps(fused):
         m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
         mods.append(m)
     graphed, eager = mods
+    o = O.DecodeOracle(w.steps + 1, w.lru_tokens, w.local_cache, 16, w.top_k_tokens, w.n_kv_heads,
+                       w.head_dim, dtype=w.dtype)
+    o.init_cache(prompt.k, prompt.v)
     inputs = DecodeInputs(w, prompt.q0, 6)
-    steps = [tuple(x.to(DEV) for x in inputs.next()) for _ in range(w.steps)]
+    host_steps = [inputs.next() for _ in range(w.steps)]
+    steps = [tuple(x.to(DEV) for x in hs) for hs in host_steps]
     xq, xk, xv = (torch.empty_like(x) for x in steps[0])
     pos = torch.tensor([w.prompt_tokens], dtype=torch.int32, device=DEV)
 
@@ -517,6 +521,7 @@ def test_graph_replay_equals_eager_steps(fused):
     a = graphed(xq, xk, xv, start_pos=pos, stage="generate")
     b = eager(*steps[0], start_pos=w.prompt_tokens, stage="generate")
     assert same(a, b)
+    check_step(graphed, o, *host_steps[0], w.prompt_tokens, a, 0, 2e-2, 1e-2)
     pos += 1
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
@@ -532,6 +537,9 @@ def test_graph_replay_equals_eager_steps(fused):
         torch.cuda.synchronize()
         assert pos.item() == w.prompt_tokens + t + 1
         assert same(out, want), f"step {t}"
+        # the replayed step against the oracle: request list, maps, times, hit mask,
+        # slot payload bit for bit, output within the bf16 tolerance
+        check_step(graphed, o, *host_steps[t], w.prompt_tokens + t, out, t, 2e-2, 1e-2)
         la, lb = graphed.lru_cache, eager.lru_cache
         assert same(la.hbm_kv_cache, lb.hbm_kv_cache), f"slots, step {t}"
         assert same(la.page_access_time, lb.page_access_time)
@@ -540,6 +548,37 @@ def test_graph_replay_equals_eager_steps(fused):
         assert la.last_miss_counts().sum().item() > 0
     c = w.prompt_tokens + w.steps - w.dram_tokens
     assert same(graphed.cache_k[0, :c], eager.cache_k[0, :c])
+
+
+def test_page_cache_path_at_32k_all_hits_matches_oracle():
+    """configs[1] through the page-cache path: the prefix equals the cache capacity, so
+    init_cache would pick the static cache; a page cache built directly over the same
+    prefix holds every page from the start, every request hits, no page moves, and
+    the step (scores, ordered top-k, LRU times, attention over all slots) matches the
+    oracle at full size."""
+    from dram_attention_amd import DRAMAttention, DummyCache, LRUCache
+
+    w = WORKLOADS["32k"]
+    steps = 6
+    prompt = make_prompt(w, 3)
+    m = DRAMAttention(steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                      w.n_kv_heads, w.head_dim, device=DEV, dtype=w.dtype)
+    m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+    assert isinstance(m.lru_cache, DummyCache)
+    S = m.dram_kv_cache_size
+    m.lru_cache = LRUCache(prompt.k[0, :S].to(DEV).transpose(0, 1), prompt.v[0, :S].to(DEV).transpose(0, 1),
+                           w.page_size, w.top_k_tokens // w.page_size, w.lru_tokens, device=DEV)
+    m._workspace = None
+    assert m.lru_cache.num_hbm_pages == m.lru_cache.num_dram_pages == 2048
+    o = O.DecodeOracle(steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                       w.n_kv_heads, w.head_dim, dtype=w.dtype)
+    o.init_cache(prompt.k, prompt.v, force_lru=True)
+    inputs = DecodeInputs(w, prompt.q0, 3)
+    for t in range(steps):
+        xq, xk, xv = inputs.next()
+        out = m(xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=w.prompt_tokens + t, stage="generate")
+        check_step(m, o, xq, xk, xv, w.prompt_tokens + t, out, t, 2e-2, 1e-2)
+        assert o.last_hit.all() and m.lru_cache.last_miss_counts().sum().item() == 0
 
 
 @pytest.mark.parametrize("full_size", [False, True])
