@@ -48,10 +48,6 @@ def parse_args():
                          "captures a whole model step, i.e. 32 attention layers, per graph)")
     ap.add_argument("--no-overlap", action="store_true",
                     help="page stream and attention serialised on one stream")
-    ap.add_argument("--layers", type=int, default=1,
-                    help="attention layers per model step, each with its own page cache and inputs "
-                         "(seed + layer); 32 with workload 128k is configs[3].  One model step per "
-                         "graph; value stays per layer: layer-steps per second")
     ap.add_argument("--force-lru", action="store_true",
                     help="workload 32k: run the page-cache path although the prefix fits the cache "
                          "(every request hits; the reference's init_cache would pick the static cache)")
@@ -67,6 +63,10 @@ def parse_args():
                     help="also time greedy decoding of a Llama-3.1-8B-shaped model (random weights, "
                          "random K/V of the workload's prompt length in every layer's page cache), "
                          "whole model step per HIP graph; 0 = skip")
+    ap.add_argument("--stack-layers", type=int, default=32,
+                    help="also time an attention-only stack of this many layers of the workload "
+                         "(configs[3] at 32 with workload 128k), pipelined and serial; 0 = skip")
+    ap.add_argument("--stack-steps", type=int, default=6, help="timed model steps of that stack")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 128 MiB device copy (reference point for HBM traffic counters)")
     return ap.parse_args()
@@ -75,19 +75,26 @@ def parse_args():
 class Layer:
     """One attention layer set up on the workload, plus the staged step inputs."""
 
-    def __init__(self, w, seed, total_steps, dev, overlap, force_lru=False):
+    def __init__(self, w, seed, total_steps, dev, overlap, force_lru=False, device_prompt=False):
         from dram_attention_amd import DRAMAttention, DummyCache, LRUCache
         from dram_attention_amd.synthetic import DecodeInputs, make_prompt
 
         self.w = w
-        prompt = make_prompt(w, seed)
-        self.prompt = prompt
         self.m = DRAMAttention(max_output_length=total_steps, lru_hbm_cache_size=w.lru_tokens,
                                local_cache_size=w.local_cache, page_size=w.page_size,
                                top_k=w.top_k_tokens, n_kv_heads=w.n_kv_heads, head_dim=w.head_dim,
                                device=dev, dtype=w.dtype)
         self.m.overlap_page_stream = overlap
-        self.m.init_cache(prompt.k.to(dev), prompt.v.to(dev))
+        if device_prompt:
+            # the workload's distributions drawn on the GPU (a 32-layer stack would spend a
+            # minute in the host generator); no CPU checker reads these layers
+            prompt = device_prompt_like(w, seed, dev)
+            self.m.init_cache(prompt.k, prompt.v)
+            prompt.k = prompt.v = None
+        else:
+            prompt = make_prompt(w, seed)
+            self.m.init_cache(prompt.k.to(dev), prompt.v.to(dev))
+        self.prompt = prompt
         if force_lru and isinstance(self.m.lru_cache, DummyCache):
             # the prefix fits the page cache, so init_cache chose the static cache; a page
             # cache built directly over the same prefix is the all-hits point of the LRU path
@@ -139,6 +146,98 @@ class Layer:
             self._step(rows[j], self.cnt[1, j:j + 1])
         self.cnt += n
         return self.out
+
+
+def device_prompt_like(w, seed, dev):
+    """make_prompt's distributions (K ~ N(0,1) x per-channel lognormal(0, 0.5), V ~ N(0,1),
+    q0 ~ N(0,1)) drawn by the GPU's generator; planted pages are left out."""
+    from dram_attention_amd.synthetic import Prompt
+
+    g = torch.Generator(device=dev).manual_seed(seed)
+    S, H, D = w.prompt_tokens, w.n_kv_heads, w.head_dim
+    q0 = torch.randn(w.n_q_heads, D, generator=g, device=dev)
+    k = torch.randn(S, H, D, generator=g, device=dev)
+    if w.channel_scale:
+        k *= torch.exp(0.5 * torch.randn(H, D, generator=g, device=dev))
+    v = torch.randn(S, H, D, generator=g, device=dev)
+    return Prompt(k.to(w.dtype)[None], v.to(w.dtype)[None], q0.cpu(), [])
+
+
+def stack_leg(w, n_layers, steps, warmup, seed, dev):
+    """configs[3]: `n_layers` independent attention layers of workload `w` stepped as one
+    model step per HIP graph, once with layer i's page stream overlapping the
+    selection (scores, top-k, LRU update) of the layers after it and once with the
+    layers strictly one after the other, on the same caches."""
+    from dram_attention_amd import AttentionStack
+
+    settle, rounds = 16, 2
+    total = settle + 2 * rounds * (steps + 1) + 6
+    layers = []
+    for li in range(n_layers):
+        layers.append(Layer(w, seed + 100 + li, total, dev, overlap=True, device_prompt=True))
+        if (li + 1) % 8 == 0:
+            print(f"bench.py: stack layer {li + 1}/{n_layers} built", file=sys.stderr, flush=True)
+    Hq, Hkv, D = w.n_q_heads, w.n_kv_heads, w.head_dim
+    qkv = torch.stack([l_.qkv for l_ in layers], dim=1).contiguous()      # (T, layers, width)
+    for l_ in layers:
+        l_.qs = l_.ks = l_.vs = l_.qkv = None
+    cnt = torch.tensor([0, w.prompt_tokens], dtype=torch.int32, device=dev)   # step, position
+
+    def model_step(stack):
+        rows = qkv.index_select(0, cnt[0:1])[0]                               # (layers, width)
+        xq = [rows[i, : Hq * D].view(1, 1, Hq, D) for i in range(n_layers)]
+        xk = [rows[i, Hq * D:(Hq + Hkv) * D].view(1, 1, Hkv, D) for i in range(n_layers)]
+        xv = [rows[i, (Hq + Hkv) * D:].view(1, 1, Hkv, D) for i in range(n_layers)]
+        out = stack.generate(xq, xk, xv, cnt[1:2])
+        cnt.add_(1)
+        return out
+
+    # Both orders run on the same caches, so they are timed in alternating rounds after
+    # the page caches have settled (the first steps after a prefill miss several
+    # times as many pages as the steady state).
+    graphs = {}
+    for name, pipelined in (("pipelined", True), ("serial", False)):
+        stack = AttentionStack([l_.m for l_ in layers], pipelined=pipelined)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model_step(stack)                     # eager: pinned mappings, workspaces
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graphs[name] = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graphs[name]):
+            model_step(stack)
+    for _ in range(settle):
+        graphs["serial"].replay()
+    torch.cuda.synchronize()
+    spent = {"pipelined": 0.0, "serial": 0.0}
+    for _ in range(rounds):
+        for name in ("pipelined", "serial"):
+            graphs[name].replay()                 # warm-up of the round
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                graphs[name].replay()
+            torch.cuda.synchronize()
+            spent[name] += time.perf_counter() - t0
+    res = {}
+    for name, dt in spent.items():
+        n = rounds * steps
+        res[name] = {"layer_steps_per_s": n * n_layers / dt, "model_steps_per_s": n / dt,
+                     "ms_per_model_step": dt / n * 1e3, "us_per_layer_step": dt / n / n_layers * 1e6}
+    misses = sum(int(l_.m.lru_cache.last_miss_counts().sum().item()) for l_ in layers) / n_layers
+    page_bytes = w.page_size * 2 * D * torch.empty(0, dtype=w.dtype).element_size()
+    return {"value": res["pipelined"]["layer_steps_per_s"], "unit": "decode steps/s per layer",
+            "layers": n_layers, "steps": rounds * steps, "settling_steps": settle,
+            "workload": f"configs[3] shape: {n_layers} independent layers of workload {w.name}, one page "
+                        f"cache each ({n_layers * w.n_kv_heads * w.n_dram_pages * page_bytes / 1e9:.1f} GB "
+                        "of pinned pages), one model step per HIP graph",
+            "pipelined": res["pipelined"], "serial": res["serial"],
+            "speedup_of_overlap": res["pipelined"]["layer_steps_per_s"] / res["serial"]["layer_steps_per_s"],
+            "distinct_misses_per_layer_last_step": misses,
+            "h2d_bytes_per_model_step": misses * n_layers * page_bytes,
+            "what": "pipelined: selection of layer i+1.. on a side stream while layer i's pages cross "
+                    "the host link; serial: the same launches on one stream"}
 
 
 def algorithmic_bytes(w, local_rows):
@@ -531,22 +630,13 @@ def main():
     torch.cuda.set_device(dev)
     w = WORKLOADS[args.workload]
     total = args.warmup + args.steps + args.profile_steps + 4
-    layers = []
-    for li in range(max(args.layers, 1)):
-        layers.append(Layer(w, args.seed + li, total, dev, overlap=not args.no_overlap,
-                            force_lru=args.force_lru))
-        if args.plain_scorer and isinstance(layers[-1].m.lru_cache, LRUCache):
-            layers[-1].m.lru_cache.top_k_selector.bounds_are_ordered = False
-        if li > 0:
-            layers[-1].prompt = None   # only layer 0 feeds the CPU baseline
-        if args.layers > 1:
-            print(f"bench.py: layer {li + 1}/{args.layers} built", file=sys.stderr, flush=True)
-    layer = layers[0]
-    n_layers = len(layers)
+    layer = Layer(w, args.seed, total, dev, overlap=not args.no_overlap, force_lru=args.force_lru)
+    if args.plain_scorer and isinstance(layer.m.lru_cache, LRUCache):
+        layer.m.lru_cache.top_k_selector.bounds_are_ordered = False
+    n_layers = 1
 
     def model_step():
-        for l_ in layers:
-            l_.step_from_device_state()
+        layer.step_from_device_state()
 
     torch.cuda.synchronize()
 
@@ -566,8 +656,7 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             model_step()
-        spg = (max(1, min(args.steps_per_graph, args.steps, Layer.MAX_STEPS_PER_GRAPH))
-               if n_layers == 1 else 1)
+        spg = max(1, min(args.steps_per_graph, args.steps, Layer.MAX_STEPS_PER_GRAPH))
         if spg > 1:
             graph_many = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph_many):
@@ -629,15 +718,13 @@ def main():
         "dtype": {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[w.dtype],
         "data": "synthetic",
         "config": {
-            "workload": f"configs[{3 if (w.name == '128k' and n_layers == 32) else WORKLOAD_INDEX[w.name]}] "
-                        f"{w.name}: {n_layers} layer{'s' if n_layers > 1 else ''}, {w.n_q_heads}q/{w.n_kv_heads}kv heads, D {w.head_dim}, "
+            "workload": f"configs[{WORKLOAD_INDEX[w.name]}] {w.name}: 1 layer, "
+                        f"{w.n_q_heads}q/{w.n_kv_heads}kv heads, D {w.head_dim}, "
                         f"{w.dram_tokens}-token prefix in pinned host DRAM ({w.n_dram_pages} pages/head), "
                         f"local {w.local_cache}, LRU {w.lru_tokens} tokens, top-k {w.top_k_tokens} tokens",
             "launch": ("eager" if args.eager else
                        f"hip-graph replay, {spg} decode steps per graph (one input fetch and one counter "
-                       f"increment per graph)" if n_layers == 1 else
-                       f"hip-graph replay, one model step ({n_layers} layer steps) per graph"),
-            "model_steps_per_s": args.steps / dt,
+                       f"increment per graph)"),
             "page_stream": "serialised" if args.no_overlap else "in the launch of the first attention pass",
             "seed": args.seed,
             "cache": type(layer.m.lru_cache).__name__,
@@ -680,7 +767,7 @@ def main():
     if args.cpu_steps > 0:
         leg("cpu_baseline", lambda: cpu_baseline(w, args.seed, args.cpu_steps, prompt=layer.prompt))
     if args.reference_shaped_steps > 3 and isinstance(layer.m.lru_cache, LRUCache):
-        del layer, layers, model_step
+        del layer, model_step
         torch.cuda.empty_cache()
 
         def ref_leg():
@@ -689,8 +776,12 @@ def main():
             return ref
 
         leg("reference_shaped_gpu", ref_leg)
+    if args.stack_layers > 1 and paged:
+        layer = model_step = None
+        torch.cuda.empty_cache()
+        leg("stack", lambda: stack_leg(w, args.stack_layers, args.stack_steps, 2, args.seed, dev))
     if args.model_decode_steps > 0:
-        layer = layers = model_step = None
+        layer = model_step = None
         torch.cuda.empty_cache()
         leg("model_decode", lambda: model_decode(w, args.model_decode_steps, args.seed, dev))
     print(json.dumps(result))

@@ -257,7 +257,8 @@ static int launch_attention(const AttnArgs &a, int dtype, int phase, int n_kv_he
   }
   if (phase & DA_PHASE_SECOND) {
     // everything in one call and no carried partial: one merge over all chunks
-    const bool all = (phase & DA_PHASE_FIRST) && !(phase & DA_PHASE_FIRST_MERGE);
+    const bool all = ((phase & DA_PHASE_FIRST) && !(phase & DA_PHASE_FIRST_MERGE)) ||
+                     (phase & DA_PHASE_MERGE_ALL);
     if (a.gather_blocks > 0) {
       // the re-assigned slots were attended while they were copied
     } else if (a.n_tchunks > 0) {
@@ -359,8 +360,12 @@ extern "C" int da_decode_attention_paged(
     DA_REQUIRE(overlap->slot_epoch && overlap->epoch && overlap->miss_slot &&
                    overlap->miss_count && overlap->miss_capacity >= 0,
                "da_decode_attention: incomplete overlap description");
-    DA_REQUIRE(overlap->phase >= 1 && overlap->phase <= 15, "da_decode_attention: bad phase %d",
+    DA_REQUIRE(overlap->phase >= 1 && overlap->phase <= 31, "da_decode_attention: bad phase %d",
                overlap->phase);
+    DA_REQUIRE(!(overlap->phase & DA_PHASE_MERGE_ALL) ||
+                   ((overlap->phase & DA_PHASE_SECOND) && !(overlap->phase & DA_PHASE_FIRST_MERGE)),
+               "da_decode_attention: DA_PHASE_MERGE_ALL goes with DA_PHASE_SECOND and without "
+               "DA_PHASE_FIRST_MERGE");
     DA_REQUIRE(!(overlap->phase & DA_PHASE_STREAM) ||
                    ((overlap->phase & DA_PHASE_FIRST) && overlap->gather_blocks >= 1),
                "da_decode_attention: DA_PHASE_STREAM goes with DA_PHASE_FIRST and gather_blocks >= 1");

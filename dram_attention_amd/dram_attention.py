@@ -28,9 +28,11 @@ class PagedPrefix:
     FIRST_MERGE folds those partial results into one (both may run next to the
     stream), SECOND (after the stream has finished) attends over the re-assigned
     slots and writes the output; FIRST | SECOND does everything at once.  With
-    STREAM the page stream itself runs inside the launch of the FIRST pass."""
+    STREAM the page stream itself runs inside the launch of the FIRST pass;
+    SECOND | MERGE_ALL is the final merge as a call of its own after FIRST (| STREAM)
+    without FIRST_MERGE."""
 
-    FIRST, SECOND, FIRST_MERGE, STREAM = 1, 2, 4, 8
+    FIRST, SECOND, FIRST_MERGE, STREAM, MERGE_ALL = 1, 2, 4, 8, 16
 
     def __init__(self, page_size: int, scratch, current_step: torch.Tensor, phase: int,
                  gather_blocks: int = 0, page_stores=None):
@@ -292,9 +294,14 @@ class DRAMAttention(torch.nn.Module):
         idx = lru.select_(xq)
         return idx, lru.update_(idx)
 
-    def attend_(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, start_pos, selected):
+    def attend_(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, start_pos, selected,
+                defer_merge: bool = False):
         """Second half of a decode step: the page stream for the misses select_ found
-        and attention over resident pages, local window and the new token."""
+        and attention over resident pages, local window and the new token.
+        ``defer_merge``: when the step's final merge is a launch of its own (page
+        stream and first pass in one launch), leave it out and return (out, merge)
+        where ``merge()`` issues it on whatever stream is current, ordered after
+        this call; ``out`` is complete only then.  Otherwise returns (out, None)."""
         bsz, seqlen, Hq, D = xq.shape
         if seqlen != 1:
             raise RuntimeError("generate handles one token per call")
@@ -315,7 +322,7 @@ class DRAMAttention(torch.nn.Module):
             decode_attention(xq[0, 0], prefix_k, prefix_v, self.cache_k[0], self.cache_v[0],
                              cache_len, xk[0, 0], xv[0, 0], workspace=self._workspace,
                              out=out[0, 0], cache_len_offset=offset)
-            return out
+            return (out, None) if defer_merge else out
 
         idx, scratch = selected
         prefix_k, prefix_v = lru.views()
@@ -350,15 +357,20 @@ class DRAMAttention(torch.nn.Module):
             stream_pages()
             # the same kernels as the concurrent order, so the same bits
             attend((P.FIRST | P.SECOND) if fused else (P.FIRST | P.FIRST_MERGE | P.SECOND))
-            return out
+            return (out, None) if defer_merge else out
         if fused:
             # page stream and first attention pass in one launch, then the merge: the
             # step stays a plain chain of launches on the caller's stream
-            decode_attention(*args, workspace=self._workspace, out=out[0, 0],
-                             cache_len_offset=offset,
-                             paged=PagedPrefix(self.page_size, scratch, lru.current_step,
-                                               P.STREAM | P.FIRST | P.SECOND, blocks,
-                                               lru.page_stores()))
+            def launch(phase):
+                decode_attention(*args, workspace=self._workspace, out=out[0, 0],
+                                 cache_len_offset=offset,
+                                 paged=PagedPrefix(self.page_size, scratch, lru.current_step,
+                                                   phase, blocks, lru.page_stores()))
+
+            if defer_merge:
+                launch(P.STREAM | P.FIRST)
+                return out, (lambda: launch(P.SECOND | P.MERGE_ALL))
+            launch(P.STREAM | P.FIRST | P.SECOND)
             return out
         # Shapes the fused stream does not take: pages stream in on a side stream
         # next to the first pass, and a tail pass covers them after the join.
@@ -372,4 +384,4 @@ class DRAMAttention(torch.nn.Module):
         attend(P.FIRST | P.FIRST_MERGE)
         main.wait_stream(side)                      # the pages have landed
         attend(P.SECOND)
-        return out
+        return (out, None) if defer_merge else out

@@ -8,8 +8,9 @@ stack the layers' queries do not depend on each other, so the first half of
 layer i+1 can run while layer i's pages are still crossing the host link: the
 link then never waits for a selection.
 
-``AttentionStack.generate`` issues the first halves on a side stream and the
-second halves on the caller's stream, tied together by one event per layer;
+``AttentionStack.generate`` issues the first halves (and the final merge of each
+layer's attention partials) on a side stream and the page stream + attention
+launches on the caller's stream, tied together by events;
 every layer runs exactly the launches it runs alone, on its own buffers, so the
 results have the same bits as stepping the layers one by one.  All streams have
 the default priority.  The step has no host synchronisation and can be
@@ -37,6 +38,7 @@ class AttentionStack(torch.nn.Module):
         self.pipelined = pipelined
         self._side = None
         self._events: List[torch.cuda.Event] = []
+        self._stream_done: List[torch.cuda.Event] = []
 
     def generate(self, xqs: Sequence[torch.Tensor], xks: Sequence[torch.Tensor],
                  xvs: Sequence[torch.Tensor], start_pos) -> List[torch.Tensor]:
@@ -55,17 +57,31 @@ class AttentionStack(torch.nn.Module):
             self._side = torch.cuda.Stream(device=dev)      # default priority
         while len(self._events) < n:
             self._events.append(torch.cuda.Event())
+        while len(self._stream_done) < n:
+            self._stream_done.append(torch.cuda.Event())
         side = self._side
+        selected_ev, streamed_ev = self._events, self._stream_done
         side.wait_stream(main)          # inputs are ready; the previous step has finished
-        selected = []
+        selected = [None] * n
         with torch.cuda.stream(side):
-            for layer, xq, ev in zip(self.layers, xqs, self._events):
-                selected.append(layer.select_(xq))
-                ev.record(side)
+            selected[0] = self.layers[0].select_(xqs[0])
+            selected_ev[0].record(side)
         outs = []
-        for layer, xq, xk, xv, sel, ev in zip(self.layers, xqs, xks, xvs, selected,
-                                              self._events):
-            main.wait_event(ev)         # this layer's miss list is complete
-            outs.append(layer.attend_(xq, xk, xv, start_pos, sel))
-        main.wait_stream(side)          # join (the last event already implies it)
+        for i, layer in enumerate(self.layers):
+            if i + 1 < n:               # the selection runs one layer ahead of the page streams
+                with torch.cuda.stream(side):
+                    selected[i + 1] = self.layers[i + 1].select_(xqs[i + 1])
+                    selected_ev[i + 1].record(side)
+            main.wait_event(selected_ev[i])     # this layer's miss list is complete
+            out, merge = layer.attend_(xqs[i], xks[i], xvs[i], start_pos, selected[i],
+                                       defer_merge=True)
+            outs.append(out)
+            if merge is not None:
+                # the final merge leaves the stream that owns the host link: the next
+                # layer's pages start moving as soon as this layer's have landed
+                streamed_ev[i].record(main)
+                with torch.cuda.stream(side):
+                    side.wait_event(streamed_ev[i])
+                    merge()
+        main.wait_stream(side)          # join: every merge has written its output
         return outs

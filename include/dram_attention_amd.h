@@ -318,6 +318,13 @@ int da_decode_attention_static(const void *q, int64_t q_head_stride, int n_q_hea
  *                          needed.  STREAM | FIRST | SECOND is a whole step in
  *                          two launches.  Same shape limits as
  *                          da_pages_gather_attend (DA_ENOTSUP otherwise).
+ *   DA_PHASE_MERGE_ALL   : together with DA_PHASE_SECOND in a call of its own, after
+ *                          a call with DA_PHASE_FIRST (and STREAM) but no
+ *                          FIRST_MERGE: there is no carried partial, the final
+ *                          merge takes every chunk.  Lets a caller issue the
+ *                          merge apart from the first pass (on another stream,
+ *                          so that the next layer's page stream need not wait
+ *                          for it) at the cost of no extra launch.
  * With two streams: FIRST | FIRST_MERGE next to the page stream, SECOND after the join.
  * FIRST | SECOND in one call (the page stream already complete) needs no
  * FIRST_MERGE.
@@ -328,6 +335,7 @@ int da_decode_attention_static(const void *q, int64_t q_head_stride, int n_q_hea
 #define DA_PHASE_SECOND 2
 #define DA_PHASE_FIRST_MERGE 4
 #define DA_PHASE_STREAM 8
+#define DA_PHASE_MERGE_ALL 16
 
 typedef struct da_paged_overlap {
   int32_t page_size;              /* tokens per slot; p_len = slots * page_size */
