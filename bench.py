@@ -479,7 +479,7 @@ def reference_shaped(w, seed, steps, dev):
     from dram_attention_amd.synthetic import DecodeInputs, make_prompt
 
     prompt = make_prompt(w, seed)
-    total = steps + 4
+    total = (steps + 4 + 63) // 64 * 64      # local cache rows divisible into equal key ranges
     m = DRAMAttention(max_output_length=total, lru_hbm_cache_size=w.lru_tokens,
                       local_cache_size=w.local_cache, page_size=w.page_size, top_k=w.top_k_tokens,
                       n_kv_heads=w.n_kv_heads, head_dim=w.head_dim, device=dev, dtype=w.dtype)
@@ -502,13 +502,63 @@ def reference_shaped(w, seed, steps, dev):
     scratch = LruScratch.allocate(Hkv, K, dev, lru.num_hbm_pages)
     misses = torch.zeros(1, dtype=torch.int64, device=dev)
 
-    def attend(q, k, v, mask=None):
+    # Attention passes: flash-attn's decode kernel splits the keys over many workgroups
+    # (flash_attn_with_kvcache).  torch-ROCm's fused attention ops do not (one call
+    # over the 32K-token prefix takes ~1.16 ms on this part, a bmm + softmax pair
+    # ~0.21 ms), so the stand-in splits the keys itself: the sequence is cut into
+    # `parts` batch entries, one fused call returns every part's output and
+    # log-sum-exp, and the parts are combined by their log-sum-exp (~0.09 ms).
+    fused_ok = w.dtype in (torch.bfloat16, torch.float16)
+    used = set()
+
+    def split_attend(q, k, v, parts, bias=None):
+        """q (Hkv, rep, D); k, v (Hkv, T, D) views; bias (T,) additive or None."""
+        T = k.shape[1]
+        kb = k.reshape(Hkv, parts, T // parts, D).transpose(0, 1)
+        vb = v.reshape(Hkv, parts, T // parts, D).transpose(0, 1)
+        qb = q[None].expand(parts, Hkv, rep, D)
+        if bias is None:
+            r = torch.ops.aten._scaled_dot_product_flash_attention(qb, kb, vb, 0.0, False, False,
+                                                                   scale=scale)
+            o, lse = r[0], r[1]
+        else:
+            bb = bias.view(parts, 1, 1, T // parts).expand(parts, Hkv, rep, T // parts).contiguous()
+            r = torch.ops.aten._scaled_dot_product_efficient_attention(qb, kb, vb, bb, True,
+                                                                       scale=scale)
+            o, lse = r[0], r[1][..., :rep]
+        lse = lse.float()
+        total = torch.logsumexp(lse, 0)
+        return (o.float() * torch.exp(lse - total)[..., None]).sum(0), total
+
+    def bmm_attend(q, k, v, mask=None):
         s_ = torch.bmm(q, k.transpose(1, 2)).float() * scale          # (Hkv, rep, T)
         if mask is not None:
             s_ = s_.masked_fill(mask, float("-inf"))
         lse = torch.logsumexp(s_, dim=-1)
         p = torch.exp(s_ - lse[..., None]).to(q.dtype)
         return torch.bmm(p, v).float(), lse
+
+    def parts_of(T, want):
+        while want > 1 and (T % want or (T // want) % 8):
+            want //= 2
+        return want
+
+    def attend(q, k, v, want_parts, beyond=None):
+        """`beyond`: bool (T,), True for rows past the valid length (device side)."""
+        if fused_ok:
+            try:
+                bias = None
+                if beyond is not None:
+                    bias = torch.zeros(k.shape[1], dtype=q.dtype, device=dev).masked_fill_(
+                        beyond, float("-inf"))
+                parts = parts_of(k.shape[1], want_parts)
+                res = split_attend(q, k, v, parts, bias)
+                used.add(f"fused op over {parts} key ranges" + (" with a length mask" if bias is not None else ""))
+                return res
+            except RuntimeError:
+                pass
+        used.add("bmm + softmax")
+        return bmm_attend(q, k, v, None if beyond is None else beyond[None, None, :])
 
     def step():
         row = qkv.index_select(0, ctr[0:1])[0]
@@ -534,13 +584,13 @@ def reference_shaped(w, seed, steps, dev):
                      max_blocks=Hkv)
         misses.add_(scratch.miss_count.sum())
         pk, pv = lru.views()
-        o_p, lse_p = attend(xq, pk, pv)
+        o_p, lse_p = attend(xq, pk, pv, 32)
         c = ctr[1:2]
         m.cache_k[0].index_copy_(0, c, xk[None])
         m.cache_v[0].index_copy_(0, c, xv[None])
         ck = m.cache_k[0].transpose(0, 1)                              # (Hkv, cap, D)
         cv = m.cache_v[0].transpose(0, 1)
-        o_s, lse_s = attend(xq, ck, cv, (rows > c)[None, None, :])
+        o_s, lse_s = attend(xq, ck, cv, 8, rows > c)
         lse = torch.logaddexp(lse_p, lse_s)
         o = o_p * torch.exp(lse_p - lse)[..., None] + o_s * torch.exp(lse_s - lse)[..., None]
         out.copy_(o.view(Hq, D))
@@ -563,10 +613,15 @@ def reference_shaped(w, seed, steps, dev):
     n = steps - 3
     return {"value": n / dt, "unit": "decode steps/s per layer", "ms_per_step": dt / n * 1e3,
             "steps": n, "distinct_misses_per_step": misses.item() / n,
+            "attention_op": "aten._scaled_dot_product_flash_attention (prefix) / _efficient_attention "
+                            "(local window), keys split over the batch axis, + log-sum-exp combine; "
+                            "paths taken: " + "; ".join(sorted(used)),
             "what": "stand-in for the reference's GPU step, not the reference: torch-ROCm ops for its "
-                    "torch/flash-attn stages (max_ip_ref scores, full argsorts, two bmm attention "
-                    "passes + log-sum-exp combine), this library's serial one-lane-per-head LRU walk "
-                    "and one-workgroup-per-head page copy for its Triton stages; launched eagerly (GPU-bound)"}
+                    "torch/flash-attn stages (max_ip_ref scores, full argsorts, two attention passes by "
+                    "torch's fused attention op with the keys split over the batch axis as flash-attn's "
+                    "decode kernel splits them, + the reference's log-sum-exp combine), this library's "
+                    "serial one-lane-per-head LRU walk and one-workgroup-per-head page copy for its "
+                    "Triton stages; launched eagerly (GPU-bound)"}
 
 
 def model_decode(w, steps, seed, dev):
