@@ -300,7 +300,14 @@ extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_i
   DA_REQUIRE(n_dram_pages <= 0x7fffffff, "da_lru_update: page ids must fit int32");
   DA_REQUIRE((flags & ~(DA_LRU_BUMP_STEP | DA_LRU_SERIAL_WALK)) == 0, "da_lru_update: unknown flags %d", flags);
   const int bump_step = (flags & DA_LRU_BUMP_STEP) ? 1 : 0;
-  const int serial = ((flags & DA_LRU_SERIAL_WALK) || k > n_hbm_pages || k > kLruMaxK) ? 1 : 0;
+  // The parallel form rests on the stamp of this call being larger than every stored
+  // access time (touched slots then sort behind all others).  With DA_LRU_BUMP_STEP
+  // the stamp is the bumped step counter, which is; a caller-supplied stamp may tie
+  // with stored times, and then only the literal walk gives the reference's result
+  // (a slot hit earlier in the walk can be chosen as a victim later in it).
+  const bool stamp_may_tie = !bump_step && n_hbm_pages <= kSelMaxK;
+  const int serial = ((flags & DA_LRU_SERIAL_WALK) || k > n_hbm_pages || k > kLruMaxK ||
+                      stamp_may_tie) ? 1 : 0;
   if (serial && n_hbm_pages > kSelMaxK)
     return fail(DA_ENOTSUP,
                 "da_lru_update: k %d > slots %d needs the serial walk, which orders at most %d "

@@ -97,8 +97,15 @@ int da_pages_build(const void *k, const void *v, int64_t tok_stride, int64_t hea
  *   minmax : (H, L, 2, D), element strides (mm_head_stride, mm_page_stride, mm_r_stride, 1)
  *   out    : (n_rows, H, L) with element strides (out_row_stride, out_head_stride, 1);
  *            out_dtype is DA_F32 or equal to `dtype`.
- * Arithmetic follows the reference kernel: for 16-bit inputs each product is
- * rounded to the input type, the maximum and the sum over D are fp32.  `flags`:
+ * Arithmetic follows the reference kernel for bf16 and fp32: for bf16 each
+ * product is rounded to bf16, the maximum and the sum over D are fp32 (Triton
+ * promotes bf16 operands of tl.maximum to fp32), fp32 is fp32 throughout.
+ * fp16 takes the bf16 scheme (products rounded to fp16, fp32 maximum and sum,
+ * one rounding at the end): a deliberate deviation.  Triton would keep fp16
+ * through the maximum AND the sum, in a reduction order it picks, which no
+ * restatement can reproduce; the reference only checks the dtype of that case
+ * (max_ip_triton_kernel_test.py:18-26), so fp16 parity is unpinned and the
+ * result here is the more accurate one.  `flags`:
  *   DA_SCORE_ROUND          : the fp32 sum is rounded to the input type before it
  *                             is stored (the value the reference ranks on, :99),
  *                             also when out_dtype is DA_F32
@@ -183,7 +190,11 @@ int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_t head_stri
  *                  gets the step value, so a later kernel can tell which slots
  *                  the page stream of this step is (still) writing
  * The end state equals the reference's serial walk for every input; K <=
- * N_hbm runs fully parallel, K > N_hbm falls back to one serial lane per head.
+ * N_hbm with DA_LRU_BUMP_STEP runs fully parallel, K > N_hbm falls back to one
+ * serial lane per head.  Without DA_LRU_BUMP_STEP the time stamp is the
+ * caller's *step and may tie with stored access times, where only the literal
+ * walk is right: such calls take it too (with more than 8192 slots they stay
+ * parallel and *step must then exceed every stored access time).
  * DA_LRU_SERIAL_WALK in `flags` takes that literal walk for any K (a checking
  * and benchmarking aid: the result is the same, only slower).
  * A miss_slot of -1 marks an entry whose slot was re-assigned later in the

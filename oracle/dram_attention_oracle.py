@@ -25,7 +25,8 @@ How each function is pinned (tests/test_oracle.py):
                       internal roundings) is PARITY UNPINNED; the closed form is the
                       contract, at the tolerance atol 2e-2 / rtol 1e-2 for bf16.
   decode geometry     lru_cache_test.py numbers; init_cache arithmetic by hand.
-The last-ulp fp32 summation order of the reference's Triton scorer is likewise
+The fp16 scorer is unpinned as well (see max_ip), and the last-ulp fp32 summation
+order of the reference's Triton scorer is likewise
 unpinned (no GPU run of it is possible here); selection parity is therefore
 stated "given identical scores".
 """
@@ -63,7 +64,12 @@ def max_ip(q: torch.Tensor, min_max: torch.Tensor) -> torch.Tensor:
     """score[n,h,l] = sum_d max(q[n,h,d]*mm[h,l,0,d], q[n,h,d]*mm[h,l,1,d]),
     returned in q.dtype (:99).  For 16-bit inputs the products are formed in the
     input type (rounded, :72,79), the maximum and the sum are fp32, and the sum is
-    rounded once on output; for fp32 everything is fp32."""
+    rounded once on output; for fp32 everything is fp32.
+    That is what Triton does for bf16 (tl.maximum promotes bf16 to fp32).  For fp16
+    Triton would stay in fp16 through the maximum and the sum, in a reduction order
+    of its choosing; this function (and the HIP kernel) use the bf16 scheme for
+    fp16 too.  PARITY UNPINNED for fp16: the reference's own test of that case
+    checks the dtype only (max_ip_triton_kernel_test.py:18-26)."""
     N, H, D = q.shape
     H1, L, R, D1 = min_max.shape
     assert H1 == H and D1 == D and R == 2

@@ -50,3 +50,16 @@ NUM_HEADS, NUM_DRAM_PAGES, NUM_HBM_PAGES, PAGE_DIM, STEP = 2, 8, 4, 64, 4
 # 0.2 -> 102 slots holding the LAST 102 pages in order; lru_hbm_cache_size=1024 -> 64 slots.
 GEOMETRY = dict(tokens=8192, page_size=16, dram_pages=512, default_hbm_pages=102,
                 hbm_pages_for_1024_tokens=64)
+
+# Not one of the reference's tests: a hand walk of its three launches
+# (dram_attention/lru_triton_kernel.py:159-194) when the caller's step EQUALS the
+# stored access times.  One head, 3 slots holding pages 3, 4, 5, all times 0, step 0,
+# requests [0, 1, 3]: the touch pass stamps slot 0 (page 3) with 0, the stable argsort
+# of [0, 0, 0] is [0, 1, 2]; the walk gives page 0 slot 0 (evicting page 3, which was
+# "hit" a moment ago), page 1 slot 1, and finds page 3 gone: a third miss, slot 2.
+STAMP_TIES = dict(
+    n_dram_pages=6, d2h=[[EMPTY, EMPTY, EMPTY, 0, 1, 2]], h2d=[[3, 4, 5]], time=[[0, 0, 0]], step=0,
+    topk=[[0, 1, 3]],
+    d2h_after=[[0, 1, EMPTY, 2, EMPTY, EMPTY]], h2d_after=[[0, 1, 3]], time_after=[[0, 0, 0]],
+    hit=[[False, False, False]], misses=[[(0, 0), (1, 1), (3, 2)]],
+)

@@ -107,6 +107,31 @@ def test_page_score_strided_query_view():
     assert same(out.cpu(), out.cpu().bfloat16().float())
 
 
+def test_page_score_fp16_follows_the_bf16_scheme():
+    """fp16 inputs: products rounded to fp16, fp32 maximum and sum, one rounding at the
+    end (the oracle's statement).  The reference's Triton kernel would accumulate in
+    fp16 in an order of its own, which nothing here can reproduce (parity unpinned,
+    its test checks the dtype only): this documents the deviation and bounds it by
+    the error of an fp16 accumulation."""
+    from dram_attention_amd import max_inner_product
+
+    N, H, D, L = 4, 2, 128, 300
+    q = torch.randn(N, H, D, generator=gen(31)).half()
+    mm = torch.randn(H, L, 2, D, generator=gen(32)).half()
+    got = max_inner_product(q.to(DEV), mm.to(DEV)).cpu()
+    assert got.dtype == torch.float16
+    want = O.max_ip(q, mm)
+    diff = (got.float() - want.float()).abs()
+    assert torch.all(diff <= want.float().abs() * 2.0 ** -10 + 1e-30)      # one fp16 step, rarely
+    assert (diff > 0).float().mean().item() < 0.02
+    # a sequential fp16 accumulation of the same rounded terms differs by far more
+    terms = torch.maximum(q[:, :, None, :] * mm[None, :, :, 0, :], q[:, :, None, :] * mm[None, :, :, 1, :])
+    acc = torch.zeros(N, H, L, dtype=torch.float16)
+    for d in range(D):
+        acc = acc + terms[..., d]
+    assert (acc.float() - want.float()).abs().max() > diff.max()
+
+
 def ordered_summaries(H, L, D, seed):
     """Random (H, L, 2, D) bf16 summaries with min <= max in every channel."""
     a = torch.randn(H, L, 2, D, generator=gen(seed)).bfloat16()
@@ -324,6 +349,52 @@ def test_load_lru_cache_reference_kats(name):
     for h, s, p in case["payload"]:
         assert same(hbm[h, s], dram[h, p])
     assert step.item() == lru_kats.STEP        # the raw function does not advance the step
+
+
+@pytest.mark.parametrize("itype,ttype", [(torch.int32, torch.int32), (torch.int64, torch.float32)])
+def test_load_lru_cache_when_the_step_ties_with_stored_times(itype, ttype):
+    """The raw function takes the caller's step as the time stamp; when it equals stored
+    access times, a slot the touch pass has just hit is still first in the eviction
+    order, and the reference's walk evicts it and pages the same page in again later
+    (hand-walked in tests/golden/lru_kats.py).  Calls without the step bump therefore
+    take the literal walk."""
+    from dram_attention_amd import load_lru_cache_
+
+    c = lru_kats.STAMP_TIES
+    dram = torch.randn(1, c["n_dram_pages"], 64, generator=gen(19)).to(DEV)
+    hbm = dram[:, 3:6].clone()
+    time = torch.tensor(c["time"], dtype=ttype, device=DEV)
+    d2h = torch.tensor(c["d2h"], dtype=itype, device=DEV)
+    h2d = torch.tensor(c["h2d"], dtype=itype, device=DEV)
+    step = torch.tensor([c["step"]], dtype=torch.int32, device=DEV)
+    load_lru_cache_(dram_kv_cache=dram, page_access_time=time,
+                    dram_page_to_hbm_page_mapping=d2h, hbm_page_to_dram_page_mapping=h2d,
+                    topk_dram_page_index=torch.tensor(c["topk"], dtype=itype, device=DEV),
+                    current_step=step, hbm_kv_cache=hbm)
+    assert d2h.cpu().tolist() == c["d2h_after"] and h2d.cpu().tolist() == c["h2d_after"]
+    assert time.cpu().float().tolist() == c["time_after"]
+    assert same(hbm[0], dram[0, [0, 1, 3]])
+    # and against the oracle on a random trace where every step repeats the stamp
+    rng = np.random.default_rng(5)
+    H, P, N, K = 3, 40, 12, 9
+    dram = torch.randn(H, P, 64, generator=gen(20))
+    st = O.LruState.initial(H, P, N)
+    hbm_o = dram[:, P - N:].clone()
+    hbm = hbm_o.to(DEV)
+    time = torch.zeros(H, N, dtype=ttype, device=DEV)
+    d2h = torch.from_numpy(st.d2h).to(itype).to(DEV)
+    h2d = torch.from_numpy(st.h2d).to(itype).to(DEV)
+    for s in (0, 0, 1, 1, 1, 3):
+        idx = rng.integers(0, P, (H, K))
+        O.lru_load(st, idx, s, dram.numpy(), hbm_o.numpy())
+        load_lru_cache_(dram_kv_cache=dram.to(DEV), page_access_time=time,
+                        dram_page_to_hbm_page_mapping=d2h, hbm_page_to_dram_page_mapping=h2d,
+                        topk_dram_page_index=torch.from_numpy(idx).to(itype).to(DEV),
+                        current_step=torch.tensor([s], dtype=torch.int32, device=DEV),
+                        hbm_kv_cache=hbm)
+        assert np.array_equal(time.cpu().numpy().astype(np.float32), st.time), f"time, stamp {s}"
+        assert np.array_equal(d2h.cpu().numpy(), st.d2h) and np.array_equal(h2d.cpu().numpy(), st.h2d)
+        assert same(hbm.cpu(), hbm_o)
 
 
 def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat16, page_dim=256,

@@ -308,3 +308,22 @@ def test_decode_oracle_lru_path_attends_over_all_resident_slots():
             p_ = torch.softmax(kk @ xq[0, 0, j].double() / math.sqrt(D), 0)
             assert torch.allclose(out[0, 0, j].double(), p_ @ vv, atol=1e-5)
         assert o.state.step == step + 1
+
+
+def test_lru_load_when_the_step_ties_with_stored_times():
+    """Hand-walked case (tests/golden/lru_kats.py STAMP_TIES): a slot hit by the touch pass
+    is still first in the eviction order when the caller's step equals the stored times,
+    so the walk evicts it and pages the same page in again later."""
+    import numpy as np
+    from tests.golden import lru_kats
+
+    c = lru_kats.STAMP_TIES
+    st = O.LruState(np.array(c["time"], dtype=np.float32), np.array(c["d2h"], dtype=np.int64),
+                    np.array(c["h2d"], dtype=np.int64), c["step"])
+    dram = np.arange(6 * 4, dtype=np.float32).reshape(1, 6, 4)
+    hbm = dram[:, 3:6].copy()
+    hit, misses = O.lru_load(st, np.array(c["topk"]), c["step"], dram, hbm)
+    assert st.d2h.tolist() == c["d2h_after"] and st.h2d.tolist() == c["h2d_after"]
+    assert st.time.tolist() == c["time_after"]
+    assert hit.tolist() == c["hit"] and [list(m) for m in misses] == c["misses"]
+    assert np.array_equal(hbm[0], dram[0, [0, 1, 3]])
