@@ -224,6 +224,12 @@ class DRAMAttention(torch.nn.Module):
         # attend over the streamed pages inside the page stream itself (when the
         # shape allows) instead of a pass over them after the stream
         self.attend_on_page_stream = True
+        # "resident": the prefix pass covers every slot of the page cache, as the
+        # reference does (dram_attention.py:195-205).  "selected": only the pages this
+        # step selected, each query head over its own list: the Quest baseline the
+        # reference compares itself with (evaluation/quest/model.py:263-316), on the
+        # same page cache and kernels.
+        self.attention_scope = "resident"
 
     def init_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor):
         """Split the prompt's (1,S,Hkv,D) keys/values into the paged prefix and the
@@ -249,6 +255,35 @@ class DRAMAttention(torch.nn.Module):
         else:
             self.lru_cache = DummyCache(k_cache=prefix_k, v_cache=prefix_v, device=self.device)
         self._workspace = None
+
+    def _attend_selected(self, xq, xk, xv, cache_len, offset, idx, out):
+        """The Quest baseline's attention (evaluation/quest/model.py:263-316): query head
+        j attends over the pages of ITS top-k list, plus the local window and the new
+        token; the two partial results are combined by their log-sum-exp.  A comparison
+        variant, not the hot path: the selected pages are gathered from their slots by
+        torch ops and the two passes are separate calls of the decode kernel."""
+        lru = self.lru_cache
+        Hq, D = xq.shape[2], xq.shape[3]
+        Hkv, K = idx.shape
+        if K > lru.num_hbm_pages:
+            raise RuntimeError("the selected-pages scope needs every selected page resident: "
+                               f"{K} requests per kv head exceed {lru.num_hbm_pages} slots")
+        lru.gather_(K)                                   # the missed pages land in their slots
+        slots = torch.gather(lru.dram_page_to_hbm_page_mapping, 1, idx)        # (Hkv, rep*kp)
+        pages = lru.hbm_kv_cache
+        sel = torch.gather(pages, 1, slots[..., None].expand(-1, -1, pages.shape[2]))
+        sel = sel.view(Hq, (K // (Hq // Hkv)) * self.page_size, 2, D)   # rows of q head h*rep + r
+        no_cache = xq.new_empty(0, Hq, D)
+        lse_p = torch.empty(Hq, dtype=torch.float32, device=xq.device)
+        lse_s = torch.empty_like(lse_p)
+        out_p = decode_attention(xq[0, 0], sel[:, :, 0], sel[:, :, 1], no_cache, no_cache, 0, None,
+                                 None, lse=lse_p)
+        out_s = decode_attention(xq[0, 0], None, None, self.cache_k[0], self.cache_v[0], cache_len,
+                                 xk[0, 0], xv[0, 0], lse=lse_s, cache_len_offset=offset)
+        lse = torch.logaddexp(lse_p, lse_s)
+        mixed = (out_p.float() * torch.exp(lse_p - lse)[:, None]
+                 + out_s.float() * torch.exp(lse_s - lse)[:, None])
+        out[0, 0].copy_(mixed)
 
     def init_cache_from_file(self, cache_dir: str, index: int) -> int:
         """init_cache from the chat example's per-layer file ``NN_cache.pth``; returns
@@ -325,6 +360,11 @@ class DRAMAttention(torch.nn.Module):
             return (out, None) if defer_merge else out
 
         idx, scratch = selected
+        if self.attention_scope == "selected":
+            self._attend_selected(xq, xk, xv, cache_len, offset, idx, out)
+            return (out, None) if defer_merge else out
+        if self.attention_scope != "resident":
+            raise RuntimeError(f"Unsupported attention scope: {self.attention_scope}")
         prefix_k, prefix_v = lru.views()
         if self._workspace is None:
             self._workspace = attention_workspace(

@@ -49,6 +49,11 @@ class ModelArgs:
     max_batch_size: int = 1
     max_seq_len: int = 2048
     dtype: torch.dtype = torch.bfloat16
+    # which of the reference's evaluated models the attention layers form:
+    #   "dram"  DRAM Attention (evaluation/dram-attention/model.py)
+    #   "quest" attention over the selected pages only (evaluation/quest/model.py:263-316)
+    #   "full"  dense attention over the whole cache (evaluation/full-attention/model.py:201-215)
+    attention_variant: str = "dram"
 
     def __post_init__(self):
         if self.n_kv_heads is None:
@@ -56,6 +61,7 @@ class ModelArgs:
         assert self.n_kv_heads <= self.n_heads
         assert self.n_heads % self.n_kv_heads == 0
         assert self.dim % self.n_heads == 0
+        assert self.attention_variant in ("dram", "quest", "full")
 
     @property
     def head_dim(self) -> int:
@@ -127,9 +133,13 @@ class Attention(nn.Module):
         self.wk = nn.Linear(args.dim, args.n_kv_heads * self.head_dim, bias=False)
         self.wv = nn.Linear(args.dim, args.n_kv_heads * self.head_dim, bias=False)
         self.wo = nn.Linear(args.n_heads * self.head_dim, args.dim, bias=False)
+        # "full": a page cache as large as the longest sequence keeps the whole prefix
+        # in HBM (init_cache then picks the static cache: plain dense attention)
+        budget = (max(args.lru_hbm_cache_size, args.max_seq_len)
+                  if args.attention_variant == "full" else args.lru_hbm_cache_size)
         self.dram_attention = DRAMAttention(
             max_output_length=args.max_output_length,
-            lru_hbm_cache_size=args.lru_hbm_cache_size,
+            lru_hbm_cache_size=budget,
             local_cache_size=args.local_cache_size,
             page_size=args.cache_page_size,
             top_k=args.cache_top_k,
@@ -138,6 +148,8 @@ class Attention(nn.Module):
             device=device,
             dtype=args.dtype,
         )
+        if args.attention_variant == "quest":
+            self.dram_attention.attention_scope = "selected"
 
     def forward(self, x: torch.Tensor, start_pos, rope_rows: torch.Tensor):
         bsz, seqlen, _ = x.shape

@@ -114,3 +114,44 @@ def test_layer_files_feed_the_model(tmp_path):
     assert c.init_cache_from_files(str(tmp_path)) == 640
     token = la.argmax(-1)
     assert torch.equal(c(token, 640), a(token, 640))
+
+
+def test_model_variants_full_and_quest():
+    """The reference's comparison models on the same kernels.  "full" keeps the whole
+    prefix in HBM behind the static cache (evaluation/full-attention/model.py:201-215):
+    its logits follow the CPU restatement of the model with a cache budget that holds
+    everything.  "quest" attends over the selected pages only
+    (evaluation/quest/model.py:263-316; the attention itself is checked against a dense
+    computation in test_gpu_module.py): here, that the model runs it in every layer and
+    that it sees fewer tokens than "dram" does."""
+    from dram_attention_amd import DummyCache, LRUCache
+
+    g = torch.Generator().manual_seed(3)
+    prompt = torch.randint(0, 257, (1, 1000), generator=g)
+    args = small_args(torch.float32, attention_variant="full")
+    model = build(args, 0)
+    oracle = M.LlamaOracle(small_args(torch.float32, lru_hbm_cache_size=1100), model.state_dict())
+    got, want = model(prompt.cuda(), 0).cpu(), oracle.forward(prompt, 0)
+    scale = want.abs().max().item()
+    pos = 1000
+    for t in range(5):
+        assert torch.allclose(got, want, atol=2e-4 * scale, rtol=1e-3), (t, (got - want).abs().max())
+        token = want.argmax(-1)
+        got, want = model(token.cuda(), pos).cpu(), oracle.forward(token, pos)
+        pos += 1
+    for layer, o in zip(model.layers, oracle.layers):
+        assert isinstance(layer.attention.dram_attention.lru_cache, DummyCache) and not o.uses_lru
+    # 8 pages per query head, 32 requests per kv head, 32 slots
+    outs = {}
+    for variant in ("dram", "quest"):
+        model = build(small_args(torch.float32, attention_variant=variant, lru_hbm_cache_size=512), 0)
+        out = model(prompt.cuda(), 0)
+        for layer in model.layers:
+            a = layer.attention.dram_attention
+            assert isinstance(a.lru_cache, LRUCache)
+            assert a.attention_scope == ("selected" if variant == "quest" else "resident")
+        outs[variant] = model(out.argmax(-1), 1000).cpu()
+        assert torch.isfinite(outs[variant]).all()
+    assert (outs["dram"] - outs["quest"]).abs().max().item() > 1e-4 * scale
+    with pytest.raises(AssertionError):
+        small_args(torch.float32, attention_variant="sparse")

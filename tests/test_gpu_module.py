@@ -550,6 +550,52 @@ def test_graph_replay_equals_eager_steps(fused):
     assert same(graphed.cache_k[0, :c], eager.cache_k[0, :c])
 
 
+def test_selected_pages_scope_matches_dense_over_the_selection():
+    """The Quest-baseline variant (evaluation/quest/model.py:263-316): query head j attends
+    over the pages of its own top-k list + local window + new token.  Checked against a
+    dense fp32 softmax over exactly those tokens, taken from the prompt by the page
+    numbers the step selected; selection and LRU state still follow the oracle (the
+    page cache works as in the default scope, only the attended set differs)."""
+    from dram_attention_amd import DRAMAttention
+
+    w = WORKLOADS["128k"].scaled(dram_tokens=16384, local_cache=1024, lru_tokens=8192,
+                                 top_k_tokens=1024, steps=5)
+    prompt = make_prompt(w, 8)
+    m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                      w.n_kv_heads, w.head_dim, device=DEV, dtype=w.dtype)
+    m.attention_scope = "selected"
+    m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+    o = O.DecodeOracle(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                       w.n_kv_heads, w.head_dim, dtype=w.dtype)
+    o.init_cache(prompt.k, prompt.v)
+    inputs = DecodeInputs(w, prompt.q0, 8)
+    S, page, rep, kp = w.dram_tokens, w.page_size, w.rep, w.pages_per_q_head
+    local_k = [prompt.k[0, S:].float()]
+    local_v = [prompt.v[0, S:].float()]
+    for t in range(w.steps):
+        xq, xk, xv = inputs.next()
+        out = m(xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=w.prompt_tokens + t, stage="generate")
+        check_step(m, o, xq, xk, xv, w.prompt_tokens + t, out, t, 2e-2, 1e-2, output=False)
+        local_k.append(xk[0].float())
+        local_v.append(xv[0].float())
+        lk, lv = torch.cat(local_k), torch.cat(local_v)                 # (rows, Hkv, D)
+        idx = m.lru_cache._topk_idx.cpu().view(w.n_kv_heads, rep, kp)
+        want = torch.empty(w.n_q_heads, w.head_dim)
+        for h in range(w.n_kv_heads):
+            for r in range(rep):
+                tok = (idx[h, r, :, None] * page + torch.arange(page)).reshape(-1)
+                k_all = torch.cat([prompt.k[0, tok, h].float(), lk[:, h]])
+                v_all = torch.cat([prompt.v[0, tok, h].float(), lv[:, h]])
+                q = xq[0, 0, h * rep + r].float()
+                p = torch.softmax(k_all @ q / math.sqrt(w.head_dim), 0)
+                want[h * rep + r] = p @ v_all
+        assert close(out[0, 0].cpu().float(), want, 2e-2, 1e-2), f"step {t}"
+    with pytest.raises(RuntimeError, match="Unsupported attention scope"):
+        m.attention_scope = "everything"
+        x = inputs.next()
+        m(x[0].to(DEV), x[1].to(DEV), x[2].to(DEV), start_pos=w.prompt_tokens + w.steps, stage="generate")
+
+
 def test_page_cache_path_at_32k_all_hits_matches_oracle():
     """configs[1] through the page-cache path: the prefix equals the cache capacity, so
     init_cache would pick the static cache; a page cache built directly over the same
