@@ -83,8 +83,8 @@ def check_hand_placed_registers(verbose: bool = False) -> None:
                 target = labels.get(m.group(1) or m.group(2))
                 if target is not None:          # a label already seen: a backward branch, i.e. a loop
                     loops.append((target, n))
-        if len(placed) != 12 or not matrix:
-            raise RuntimeError(f"{name}: expected 12 hand-placed destinations and some MFMAs, "
+        if len(placed) != 8 or not matrix:
+            raise RuntimeError(f"{name}: expected 8 hand-placed destinations and some MFMAs, "
                                f"found {len(placed)} and {len(matrix)} registers")
         # A register may serve both only when every MFMA that names it comes after
         # the last hand-placed write to it (the variable behind it is dead by then),

@@ -7,17 +7,19 @@
 // plain vector form needs ~2.5 vector instructions per (channel, query row)
 // product pair and is bound by instruction issue at half the memory rate; this
 // form needs one per product plus a sixth of one:
-//   - the bound is picked on the packed words (v_bfi_b32 with a per-lane mask of
-//     the query's signs: one instruction per two channels);
-//   - each product is one v_dot2_f32_bf16 against (q, 0) or (0, q): a bf16 x bf16
-//     product is exact in fp32, so it equals the fp32 multiply of the unpacked
-//     operands (checked on the hardware for every pair of bf16 values, denormals
-//     included).  Operands that are not finite: 0 * inf = NaN leaks from one
-//     half of a word into the other half's product, and the plain form takes
-//     the maximum of two products as fmax does (a NaN product loses against
-//     the other one, as in the reference's tl.maximum), where this form has
-//     only one product.  Both differences can only turn a score into NaN,
-//     never into another number, so a NaN score is recomputed the plain way;
+//   - min and max words are interleaved once per page slice (v_perm_b32: a word
+//     (max_d, min_d) per channel, shared by all query rows), and the query is
+//     split by sign into (q+, q-) words with q+ = q where q >= 0 else 0 and
+//     q- = q - q+.  One v_dot2_f32_bf16 then gives max_d*q+ + min_d*q-, which
+//     is q * (q >= 0 ? max : min) with an added +-0: a bf16 x bf16 product is
+//     exact in fp32, so this equals the fp32 multiply of the unpacked operands
+//     (checked on the hardware for every pair of bf16 values, denormals
+//     included).  Operands that are not finite: 0 * inf = NaN arises from the
+//     bound that should not count, and the plain form takes the maximum of
+//     two products as fmax does (a NaN product loses against the other one,
+//     as in the reference's tl.maximum), where this form has only their sum.
+//     Both differences can only turn a score into NaN, never into another
+//     number, so a NaN score is recomputed the plain way;
 //   - two products are rounded by one v_cvt_pk_bf16_f32, and the packed words
 //     ARE the A operand of v_mfma_f32_16x16x32_bf16: the matrix core adds up the
 //     8 products of a lane and the 4 lanes that share a row in fp32, which takes
@@ -46,14 +48,11 @@ typedef float score_f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 score_bf16x8 __attribute__((ext_vector_type(8)));
 typedef short score_i16x2 __attribute__((ext_vector_type(2)));
 
-// The products of one 16-byte slice (4 packed words = 8 channels) with one query
-// row, as a block of hand-placed instructions:
-//   v_bfi_b32       sel = (pick & max) | (~pick & min): the bound each channel needs
-//   v_dot2_f32_bf16 lo = sel.lo*q.lo + sel.hi*0, hi = sel.lo*0 + sel.hi*q.hi, in the
-//                   three-operand encoding with a literal zero addend (the
-//                   compiler's own choice, the accumulating two-operand form,
-//                   costs a register clear per product, and it splits half of
-//                   the bitfield picks into two instructions)
+// The products of one 16-byte slice (4 channel pairs = 8 channels) with one query
+// row, as a block of hand-placed instructions: lo[e] = max*q+ + min*q- of the even
+// channel of pair e, hi[e] of the odd one, each one v_dot2_f32_bf16 in the
+// three-operand encoding with a literal zero addend (the compiler's own choice,
+// the accumulating two-operand form, costs a register clear per product).
 // Inline asm is invisible to the compiler's hazard tracking, so the block keeps
 // two rules by construction:
 //   - a dot product's result may be read by another kind of vector instruction
@@ -63,29 +62,24 @@ typedef short score_i16x2 __attribute__((ext_vector_type(2)));
 //     in flight still reads as its addend or is about to write: the block
 //     writes ONLY read-write operands, variables that stay live for the whole
 //     kernel, which the register allocator therefore never hands to an MFMA.
-__device__ __forceinline__ void slice_products(uint32_t (&sel)[4], uint32_t (&lo)[4],
-                                               uint32_t (&hi)[4], const uint32_t (&pick)[4],
-                                               const u32x4 &vmax, const u32x4 &vmin,
-                                               const uint32_t (&qlo)[4], const uint32_t (&qhi)[4]) {
-  asm("v_bfi_b32 %0, %12, %16, %20\n\t"
-      "v_bfi_b32 %1, %13, %17, %21\n\t"
-      "v_bfi_b32 %2, %14, %18, %22\n\t"
-      "v_bfi_b32 %3, %15, %19, %23\n\t"
-      "v_dot2_f32_bf16 %4, %0, %24, 0\n\t"
-      "v_dot2_f32_bf16 %8, %0, %28, 0\n\t"
-      "v_dot2_f32_bf16 %5, %1, %25, 0\n\t"
-      "v_dot2_f32_bf16 %9, %1, %29, 0\n\t"
-      "v_dot2_f32_bf16 %6, %2, %26, 0\n\t"
-      "v_dot2_f32_bf16 %10, %2, %30, 0\n\t"
-      "v_dot2_f32_bf16 %7, %3, %27, 0\n\t"
-      "v_dot2_f32_bf16 %11, %3, %31, 0\n\t"
+__device__ __forceinline__ void slice_products(uint32_t (&lo)[4], uint32_t (&hi)[4],
+                                               const u32x4 &even, const u32x4 &odd,
+                                               const uint32_t (&q_even)[4],
+                                               const uint32_t (&q_odd)[4]) {
+  asm("v_dot2_f32_bf16 %0, %8, %16, 0\n\t"
+      "v_dot2_f32_bf16 %4, %12, %20, 0\n\t"
+      "v_dot2_f32_bf16 %1, %9, %17, 0\n\t"
+      "v_dot2_f32_bf16 %5, %13, %21, 0\n\t"
+      "v_dot2_f32_bf16 %2, %10, %18, 0\n\t"
+      "v_dot2_f32_bf16 %6, %14, %22, 0\n\t"
+      "v_dot2_f32_bf16 %3, %11, %19, 0\n\t"
+      "v_dot2_f32_bf16 %7, %15, %23, 0\n\t"
       "s_nop 2"
-      : "+v"(sel[0]), "+v"(sel[1]), "+v"(sel[2]), "+v"(sel[3]), "+v"(lo[0]), "+v"(lo[1]),
-        "+v"(lo[2]), "+v"(lo[3]), "+v"(hi[0]), "+v"(hi[1]), "+v"(hi[2]), "+v"(hi[3])
-      : "v"(pick[0]), "v"(pick[1]), "v"(pick[2]), "v"(pick[3]), "v"(vmax[0]), "v"(vmax[1]),
-        "v"(vmax[2]), "v"(vmax[3]), "v"(vmin[0]), "v"(vmin[1]), "v"(vmin[2]), "v"(vmin[3]),
-        "v"(qlo[0]), "v"(qlo[1]), "v"(qlo[2]), "v"(qlo[3]), "v"(qhi[0]), "v"(qhi[1]),
-        "v"(qhi[2]), "v"(qhi[3]));
+      : "+v"(lo[0]), "+v"(lo[1]), "+v"(lo[2]), "+v"(lo[3]), "+v"(hi[0]), "+v"(hi[1]),
+        "+v"(hi[2]), "+v"(hi[3])
+      : "v"(even[0]), "v"(even[1]), "v"(even[2]), "v"(even[3]), "v"(odd[0]), "v"(odd[1]),
+        "v"(odd[2]), "v"(odd[3]), "v"(q_even[0]), "v"(q_even[1]), "v"(q_even[2]),
+        "v"(q_even[3]), "v"(q_odd[0]), "v"(q_odd[1]), "v"(q_odd[2]), "v"(q_odd[3]));
 }
 
 // The plain statement of one score (any non-finite operand behaves as in the
@@ -127,12 +121,10 @@ page_score_tile_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t
 
   // The only registers the inline asm ever writes (see slice_products), claimed
   // before anything else so that they are never shared with an MFMA operand.
-  uint32_t t_sel[4], t_lo[4], t_hi[4];
+  uint32_t t_lo[4], t_hi[4];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0\n\tv_mov_b32 %2, 0"
-                 : "=v"(t_sel[e]), "=v"(t_lo[e]), "=v"(t_hi[e]));
-  }
+  for (int e = 0; e < 4; ++e)
+    asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0" : "=v"(t_lo[e]), "=v"(t_hi[e]));
 
   // the query words of this lane's 8 channels, requested first and unpacked only
   // after the first round's page loads have gone out (loads complete in order)
@@ -142,19 +134,20 @@ page_score_tile_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t
     const int n = row0 + r < n_rows ? row0 + r : n_rows - 1;
     qw[r] = load16(q + (n * q_row_stride + h * q_head_stride + (int64_t)chunk * 8) * 2);
   }
-  // query operands: (q, 0) and (0, q) words for the two products of a pair, and
-  // the sign mask that picks max (q >= 0) or min
-  uint32_t qlo[kRows][4], qhi[kRows][4], pick[kRows][4];
+  // query operands: per channel pair the words (q+, q-) of its even and of its odd
+  // channel, q+ = q where its sign bit is clear else 0, q- = q - q+
+  uint32_t q_even[kRows][4], q_odd[kRows][4];
   auto unpack_query = [&]() {
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const uint32_t word = qw[r][e];
-        qlo[r][e] = word & 0x0000ffffu;
-        qhi[r][e] = word & 0xffff0000u;
-        // each half: all ones when its sign bit is clear (packed arithmetic shift, then not)
-        pick[r][e] = ~__builtin_bit_cast(uint32_t, __builtin_bit_cast(score_i16x2, word) >> 15);
+        // each half: all ones when its sign bit is set (packed arithmetic shift)
+        const uint32_t neg_mask = __builtin_bit_cast(uint32_t, __builtin_bit_cast(score_i16x2, word) >> 15);
+        const uint32_t pos = word & ~neg_mask, neg = word & neg_mask;
+        q_even[r][e] = __builtin_amdgcn_perm(neg, pos, 0x05040100u);   // (pos.lo, neg.lo)
+        q_odd[r][e] = __builtin_amdgcn_perm(neg, pos, 0x07060302u);    // (pos.hi, neg.hi)
       }
     }
   };
@@ -195,9 +188,16 @@ page_score_tile_kernel(const char *__restrict__ q, int64_t q_row_stride, int64_t
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const int s = s4 + t;
+        // (max_d, min_d) words of the even and of the odd channel of every pair
+        u32x4 even, odd;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          even[e] = __builtin_amdgcn_perm(vmin[s][e], vmax[s][e], 0x05040100u);
+          odd[e] = __builtin_amdgcn_perm(vmin[s][e], vmax[s][e], 0x07060302u);
+        }
 #pragma unroll
         for (int r = 0; r < kRows; ++r) {
-          slice_products(t_sel, t_lo, t_hi, pick[r], vmax[s], vmin[s], qlo[r], qhi[r]);
+          slice_products(t_lo, t_hi, even, odd, q_even[r], q_odd[r]);
           u32x4 b;
 #pragma unroll
           for (int e = 0; e < 4; ++e) b[e] = pack_bf16(as_f32(t_lo[e]), as_f32(t_hi[e]));
