@@ -794,6 +794,9 @@ def main():
                       if w.dtype != torch.float32 else "decode_attention_split_kernel (fp32, vector units)",
             "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
+            "traffic_source": ("not measured by this run: FETCH_SIZE x 2.0 + WRITE_SIZE per launch of this kernel "
+                               "from the committed counter runs, profiles/bench_128k_hbm_traffic_pmc.md"
+                               if traffic is not None else None),
             "algorithmic_bytes": attn_b, "avg_us": attn_us,
         },
         "kernels_us": kernel_us,
