@@ -18,6 +18,7 @@ import torch.nn.functional as F
 from . import _lib
 from .lru_cache import DummyCache, LRUCache
 from .lru_kernel import GATHER_BLOCKS, gather_attend_supported
+from .topk_selector import TokenMaxTopKSelector
 
 
 class PagedPrefix:
@@ -230,6 +231,11 @@ class DRAMAttention(torch.nn.Module):
         # reference compares itself with (evaluation/quest/model.py:263-316), on the
         # same page cache and kernels.
         self.attention_scope = "resident"
+        # "bound": pages ranked by the min/max upper bound (topk_selector.py:37-61 of the
+        # reference).  "token_max": by the best token of each page, the accuracy ceiling
+        # of page selection (evaluation/quest-top-k-oracle/model.py:267-275); keeps all
+        # prefix keys on the device.  Read by init_cache.
+        self.page_selector = "bound"
 
     def init_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor):
         """Split the prompt's (1,S,Hkv,D) keys/values into the paged prefix and the
@@ -252,6 +258,11 @@ class DRAMAttention(torch.nn.Module):
                 lru_hbm_cache_size=self.lru_hbm_cache_size,
                 device=self.device,
             )
+            if self.page_selector == "token_max":
+                self.lru_cache.top_k_selector = TokenMaxTopKSelector(
+                    prefix_k, self.lru_cache.num_dram_pages, device=self.device)
+            elif self.page_selector != "bound":
+                raise RuntimeError(f"Unsupported page selector: {self.page_selector}")
         else:
             self.lru_cache = DummyCache(k_cache=prefix_k, v_cache=prefix_v, device=self.device)
         self._workspace = None

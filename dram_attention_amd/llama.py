@@ -52,6 +52,8 @@ class ModelArgs:
     # which of the reference's evaluated models the attention layers form:
     #   "dram"  DRAM Attention (evaluation/dram-attention/model.py)
     #   "quest" attention over the selected pages only (evaluation/quest/model.py:263-316)
+    #   "quest_oracle" the same with pages ranked by their best token instead of the
+    #           min/max bound (evaluation/quest-top-k-oracle/model.py:267-275)
     #   "full"  dense attention over the whole cache (evaluation/full-attention/model.py:201-215)
     attention_variant: str = "dram"
 
@@ -61,7 +63,7 @@ class ModelArgs:
         assert self.n_kv_heads <= self.n_heads
         assert self.n_heads % self.n_kv_heads == 0
         assert self.dim % self.n_heads == 0
-        assert self.attention_variant in ("dram", "quest", "full")
+        assert self.attention_variant in ("dram", "quest", "quest_oracle", "full")
 
     @property
     def head_dim(self) -> int:
@@ -148,8 +150,10 @@ class Attention(nn.Module):
             device=device,
             dtype=args.dtype,
         )
-        if args.attention_variant == "quest":
+        if args.attention_variant in ("quest", "quest_oracle"):
             self.dram_attention.attention_scope = "selected"
+        if args.attention_variant == "quest_oracle":
+            self.dram_attention.page_selector = "token_max"
 
     def forward(self, x: torch.Tensor, start_pos, rope_rows: torch.Tensor):
         bsz, seqlen, _ = x.shape

@@ -130,3 +130,32 @@ class IPUpperboundTopKSelector:
         if out is None:
             out = torch.empty(H, seq_len * rep * k, dtype=torch.int64, device=q.device)
         return topk_pages(scores, rep, k, out, rep * k, seq_len * rep * k, k, lru=lru)
+
+
+class TokenMaxTopKSelector(IPUpperboundTopKSelector):
+    """Ranks pages by their best token: score = max over the page's tokens of q.k, the
+    quantity the min/max bound estimates from above.  The selector of the reference's
+    accuracy ceiling for page selection (evaluation/quest-top-k-oracle/model.py:267-275);
+    a comparison variant, not the hot path: it keeps every prefix key on the device and
+    scores with torch ops in the input type, as that model does.  Ranking, tie order
+    and the LRU-side layout are the parent's (the same top-k kernel)."""
+
+    def __init__(self, k_cache: torch.Tensor, num_pages: int, device="cuda"):
+        super().__init__(k_cache, num_pages, device=device)
+        num_heads, length, head_dim = k_cache.shape
+        self._paged_keys = k_cache.to(device=device).contiguous().view(
+            num_heads, num_pages, length // num_pages, head_dim)
+
+    def scores(self, q: torch.Tensor) -> torch.Tensor:
+        bsz, seq_len, num_q_heads, head_dim = q.shape
+        assert bsz == 1, f"Only batch size 1 is supported, but got batch size {bsz}"
+        assert num_q_heads % self.num_kv_heads == 0
+        rep = num_q_heads // self.num_kv_heads
+        H, L = self.num_kv_heads, self._paged_keys.shape[1]
+        n_rows = seq_len * rep
+        if self._scores is None or self._scores.shape[0] != n_rows:
+            self._scores = torch.empty(n_rows, H, L, dtype=torch.float32, device=q.device)
+        qv = q[0].view(seq_len, H, rep, head_dim)
+        best = torch.einsum("hptd,shrd->srhpt", self._paged_keys, qv).amax(dim=-1)
+        self._scores.copy_(best.reshape(n_rows, H, L))
+        return self._scores

@@ -116,15 +116,18 @@ def test_layer_files_feed_the_model(tmp_path):
     assert torch.equal(c(token, 640), a(token, 640))
 
 
-def test_model_variants_full_and_quest():
+def test_model_variants_full_quest_and_quest_oracle():
     """The reference's comparison models on the same kernels.  "full" keeps the whole
     prefix in HBM behind the static cache (evaluation/full-attention/model.py:201-215):
     its logits follow the CPU restatement of the model with a cache budget that holds
     everything.  "quest" attends over the selected pages only
     (evaluation/quest/model.py:263-316; the attention itself is checked against a dense
     computation in test_gpu_module.py): here, that the model runs it in every layer and
-    that it sees fewer tokens than "dram" does."""
+    that it sees fewer tokens than "dram" does.  "quest_oracle" is "quest" with pages
+    ranked by their best token (evaluation/quest-top-k-oracle/model.py:267-275; the
+    selector is checked in test_gpu_module.py)."""
     from dram_attention_amd import DummyCache, LRUCache
+    from dram_attention_amd.topk_selector import TokenMaxTopKSelector
 
     g = torch.Generator().manual_seed(3)
     prompt = torch.randint(0, 257, (1, 1000), generator=g)
@@ -143,13 +146,14 @@ def test_model_variants_full_and_quest():
         assert isinstance(layer.attention.dram_attention.lru_cache, DummyCache) and not o.uses_lru
     # 8 pages per query head, 32 requests per kv head, 32 slots
     outs = {}
-    for variant in ("dram", "quest"):
+    for variant in ("dram", "quest", "quest_oracle"):
         model = build(small_args(torch.float32, attention_variant=variant, lru_hbm_cache_size=512), 0)
         out = model(prompt.cuda(), 0)
         for layer in model.layers:
             a = layer.attention.dram_attention
             assert isinstance(a.lru_cache, LRUCache)
-            assert a.attention_scope == ("selected" if variant == "quest" else "resident")
+            assert a.attention_scope == ("resident" if variant == "dram" else "selected")
+            assert isinstance(a.lru_cache.top_k_selector, TokenMaxTopKSelector) == (variant == "quest_oracle")
         outs[variant] = model(out.argmax(-1), 1000).cpu()
         assert torch.isfinite(outs[variant]).all()
     assert (outs["dram"] - outs["quest"]).abs().max().item() > 1e-4 * scale

@@ -596,6 +596,45 @@ def test_selected_pages_scope_matches_dense_over_the_selection():
         m(x[0].to(DEV), x[1].to(DEV), x[2].to(DEV), start_pos=w.prompt_tokens + w.steps, stage="generate")
 
 
+def test_token_max_selector_ranks_pages_by_their_best_token():
+    """The page selector of the reference's accuracy ceiling
+    (evaluation/quest-top-k-oracle/model.py:267-275): score = max over the page's tokens
+    of q.k.  Checked against a brute-force fp32 computation from the prompt's keys and
+    against the property that makes Quest's bound a bound (best token <= min/max score,
+    page by page); ranking, LRU state and payload then follow the oracle fed with
+    these scores, and the attended set is each query head's own list."""
+    from dram_attention_amd import DRAMAttention
+    from dram_attention_amd.topk_selector import TokenMaxTopKSelector
+
+    w = WORKLOADS["128k"].scaled(dram_tokens=8192, local_cache=512, lru_tokens=4096,
+                                 top_k_tokens=512, steps=4)
+    prompt = make_prompt(w, 11)
+    m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                      w.n_kv_heads, w.head_dim, device=DEV, dtype=w.dtype)
+    m.attention_scope = "selected"
+    m.page_selector = "token_max"
+    m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+    assert isinstance(m.lru_cache.top_k_selector, TokenMaxTopKSelector)
+    o = O.DecodeOracle(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                       w.n_kv_heads, w.head_dim, dtype=w.dtype)
+    o.init_cache(prompt.k, prompt.v)
+    inputs = DecodeInputs(w, prompt.q0, 11)
+    S, page, rep = w.dram_tokens, w.page_size, w.rep
+    keys = prompt.k[0, :S].float().view(S // page, page, w.n_kv_heads, w.head_dim)
+    for t in range(w.steps):
+        xq, xk, xv = inputs.next()
+        out = m(xq.to(DEV), xk.to(DEV), xv.to(DEV), start_pos=w.prompt_tokens + t, stage="generate")
+        q = xq[0, 0].float().view(w.n_kv_heads, rep, w.head_dim)
+        best = torch.einsum("pthd,hrd->rhpt", keys, q).amax(-1)          # (rep, Hkv, P)
+        bound = O.scores_for_selection(xq, o.min_max)
+        assert torch.all(best <= bound + bound.abs() * 2.0 ** -6 + 1e-3), f"bound, step {t}"
+        check_step(m, o, xq, xk, xv, w.prompt_tokens + t, out, t, 2e-2, 1e-2, output=False,
+                   own_scores=best)
+    m.page_selector = "best_guess"
+    with pytest.raises(RuntimeError, match="Unsupported page selector"):
+        m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+
+
 def test_page_cache_path_at_32k_all_hits_matches_oracle():
     """configs[1] through the page-cache path: the prefix equals the cache capacity, so
     init_cache would pick the static cache; a page cache built directly over the same
