@@ -400,17 +400,25 @@ __device__ __forceinline__ StreamRange stream_range(int b, int n_blocks, int64_t
   return {b * total / n_eff, (b + 1) * total / n_eff};
 }
 
-inline int pick_chunk(int64_t total_tokens, int n_kv_heads, int step_tokens) {
+inline int pick_chunk(int64_t p_len, int64_t c_capacity, int n_kv_heads, int step_tokens) {
   // ~2 blocks per CU on a 256-CU part: every block pays a fixed prologue and a
   // merge epilogue, so few long chunks beat many short ones (measured on the
   // 128K workload: 31.9 us at 512 blocks, 32.6 us at 2048); never below one
   // unrolled round.
   const int64_t want_blocks = 256 * 2;
-  int64_t chunk = total_tokens * n_kv_heads / want_blocks;
+  int64_t chunk = (p_len + c_capacity) * n_kv_heads / want_blocks;
   const int round = step_tokens * kAttnUnroll;
   if (chunk < round) chunk = round;
   if (chunk > 4096) chunk = 4096;
-  return (int)(ceil_div(chunk, round) * round);
+  chunk = ceil_div(chunk, round) * round;
+  // The two segments are cut separately, so each may add a short last chunk, and a
+  // few blocks beyond what the part holds at once run as a second round behind
+  // all the others (128K workload: 65 chunks x 8 heads = 520 blocks of 576 tokens
+  // take 28.6 us, 59 x 8 = 472 blocks of 640 tokens 26.4 us).
+  while (chunk < 4096 &&
+         (ceil_div(p_len, chunk) + ceil_div(c_capacity, chunk)) * n_kv_heads > want_blocks)
+    chunk += round;
+  return (int)chunk;
 }
 
 inline int lanes_of(int head_dim, int dtype) {
@@ -436,7 +444,7 @@ inline ChunkPlan plan_chunks(int n_kv_heads, int lanes, int64_t p_len, int64_t c
                              int64_t miss_tokens) {
   const int step_tokens = kAttnWaves * (64 / lanes);
   ChunkPlan p;
-  p.chunk = pick_chunk(p_len + c_capacity, n_kv_heads, step_tokens);
+  p.chunk = pick_chunk(p_len, c_capacity, n_kv_heads, step_tokens);
   p.n_p = (int)ceil_div(p_len, p.chunk);
   p.n_l = (int)ceil_div(c_capacity, p.chunk);
   // the tail is short and every block starts with a dependent slot lookup:
