@@ -57,7 +57,8 @@ SIGNATURES = {
     "da_topk_pages_lru": (
         c_int,
         [c_void_p, c_int64, c_int64, c_int, c_int, c_int, c_int64, c_int, c_void_p, c_int64,
-         c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p],
+         c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p,
+         c_size_t, c_void_p],
     ),
     "da_pages_gather": (
         c_int,

@@ -135,7 +135,7 @@ def lru_candidates(page_access_time: torch.Tensor, scratch: LruScratch) -> torch
         _lib.load().da_topk_pages_lru(
             None, 0, 0, 0, 1, H, 0, 0, None, 0, 0, 0, _lib.itype_code(torch.int64),
             page_access_time.data_ptr(), page_access_time.stride(0),
-            _lib.time_code(page_access_time.dtype), N, cand.shape[1], cand.data_ptr(),
+            _lib.time_code(page_access_time.dtype), N, cand.shape[1], cand.data_ptr(), None, 0,
             _lib.stream_ptr(page_access_time.device)),
         "da_topk_pages_lru")
     return cand

@@ -34,16 +34,38 @@ def page_min_max(k_cache: torch.Tensor, num_pages: int) -> torch.Tensor:
     return out
 
 
+_split_workspaces = {}
+
+
+def _split_workspace(n_rows: int, n_heads: int, n_pages: int, k: int, device) -> torch.Tensor | None:
+    """Candidate buffer of the two-launch selection of long rows (None: not needed).
+    One buffer per shape and device, kept between calls: launches of one stream
+    follow each other, and the buffer carries nothing from call to call."""
+    need = _lib.load().da_topk_pages_workspace_bytes(n_rows, n_heads, n_pages, k)
+    if need == 0:
+        return None
+    key = (n_rows, n_heads, n_pages, k, str(device), torch.cuda.current_stream(device).cuda_stream)
+    ws = _split_workspaces.get(key)
+    if ws is None:
+        ws = _split_workspaces[key] = torch.empty(need, dtype=torch.uint8, device=device)
+    return ws
+
+
 def topk_pages(scores: torch.Tensor, rep: int, k: int, out: torch.Tensor,
-               seq_stride: int, head_stride: int, rep_stride: int, lru=None) -> torch.Tensor:
+               seq_stride: int, head_stride: int, rep_stride: int, lru=None,
+               workspace: torch.Tensor | None = None) -> torch.Tensor:
     """Ordered top-k of every row of fp32 ``scores`` (n_rows, H, L); row n of head h
     lands at (n // rep)*seq_stride + h*head_stride + (n % rep)*rep_stride in ``out``.
     ``lru`` = (page_access_time (H, N), candidates (H, k_cand) int32): the same launch
     also lists the k_cand least recently used slots of every head, for the LRU
-    update that follows."""
+    update that follows.  ``workspace``: candidate buffer for rows longer than
+    16384 pages (da_topk_pages_workspace_bytes); by default one per shape and stream
+    is kept by this module."""
     n_rows, H, L = scores.shape
     assert scores.dtype == torch.float32 and (L <= 1 or scores.stride(-1) == 1)
     lib = _lib.load()
+    if workspace is None and n_rows > 0 and k > 0 and L > 16384:
+        workspace = _split_workspace(n_rows, H, L, k, scores.device)
     if lru is None:
         time_ptr, time_hs, time_code, n_slots, k_cand, cand_ptr = None, 0, 0, 0, 0, None
     else:
@@ -58,6 +80,8 @@ def topk_pages(scores: torch.Tensor, rep: int, k: int, out: torch.Tensor,
             scores.data_ptr(), scores.stride(0), scores.stride(1), n_rows, rep, H, L, k,
             out.data_ptr(), seq_stride, head_stride, rep_stride, _lib.itype_code(out.dtype),
             time_ptr, time_hs, time_code, n_slots, k_cand, cand_ptr,
+            None if workspace is None else workspace.data_ptr(),
+            0 if workspace is None else workspace.numel() * workspace.element_size(),
             _lib.stream_ptr(scores.device),
         ),
         "da_topk_pages",
@@ -86,6 +110,7 @@ class IPUpperboundTopKSelector:
         # contents into chunk_min_max
         self.bounds_are_ordered = True
         self._scores = None
+        self._split_ws = {}     # candidate buffers of long rows, by (rows, k): this selector's own
 
     def scores(self, q: torch.Tensor) -> torch.Tensor:
         """fp32 scores (seq_len*rep, num_kv_heads, num_pages); row s*rep + r is query
@@ -108,6 +133,14 @@ class IPUpperboundTopKSelector:
         return page_scores(qv, self.chunk_min_max, self._scores, round_to_input=True,
                            ordered_bounds=self.bounds_are_ordered)
 
+    def _workspace(self, scores: torch.Tensor, k: int):
+        n_rows, H, L = scores.shape
+        if (n_rows, k) not in self._split_ws:
+            need = _lib.load().da_topk_pages_workspace_bytes(n_rows, H, L, k)
+            self._split_ws[(n_rows, k)] = (torch.empty(need, dtype=torch.uint8, device=scores.device)
+                                           if need else None)
+        return self._split_ws[(n_rows, k)]
+
     def top_k(self, q: torch.Tensor, k: int) -> torch.Tensor:
         """Indices of the top k pages, (seq_len, num_kv_heads, rep, k) int64, best first."""
         bsz, seq_len, num_q_heads, _ = q.shape
@@ -116,7 +149,8 @@ class IPUpperboundTopKSelector:
         H, L = self.num_kv_heads, scores.shape[-1]
         k = min(k, L)
         out = torch.empty(seq_len, H, rep, k, dtype=torch.int64, device=q.device)
-        return topk_pages(scores, rep, k, out, H * rep * k, rep * k, k)
+        return topk_pages(scores, rep, k, out, H * rep * k, rep * k, k,
+                          workspace=self._workspace(scores, k))
 
     def top_k_for_lru(self, q: torch.Tensor, k: int, out: torch.Tensor | None = None, lru=None):
         """The same selection laid out as the LRU consumes it, (num_kv_heads,
@@ -129,7 +163,8 @@ class IPUpperboundTopKSelector:
         k = min(k, L)
         if out is None:
             out = torch.empty(H, seq_len * rep * k, dtype=torch.int64, device=q.device)
-        return topk_pages(scores, rep, k, out, rep * k, seq_len * rep * k, k, lru=lru)
+        return topk_pages(scores, rep, k, out, rep * k, seq_len * rep * k, k, lru=lru,
+                          workspace=self._workspace(scores, k))
 
 
 class TokenMaxTopKSelector(IPUpperboundTopKSelector):

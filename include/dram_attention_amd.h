@@ -138,7 +138,11 @@ int da_page_score(const void *q, int64_t q_row_stride, int64_t q_head_stride,
  *            (n / rep)*out_seq_stride + h*out_head_stride + (n % rep)*out_rep_stride
  * Order: descending score; equal scores by ascending page index (a stable
  * descending sort).  -0.0 equals +0.0; NaN ranks above +inf (torch's order).
- * workspace: da_topk_pages_workspace_bytes(...) bytes, no initial state needed.
+ * workspace: da_topk_pages_workspace_bytes(...) bytes (0 for rows of up to 16384
+ * pages), no initial state needed.  Longer rows are cut into parts that one
+ * workgroup each reduces to kp candidates, and a second launch selects among the
+ * candidates (same result, ties included); without a workspace of that size
+ * (NULL is allowed) one workgroup per row walks the whole row instead.
  */
 size_t da_topk_pages_workspace_bytes(int n_rows, int n_heads, int64_t n_pages, int kp);
 int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
@@ -162,7 +166,8 @@ int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_t head_stri
                       void *out, int64_t out_seq_stride, int64_t out_head_stride,
                       int64_t out_rep_stride, int out_itype, const void *access_time,
                       int64_t time_head_stride, int time_type, int n_hbm_pages, int k_cand,
-                      int32_t *candidates, void *stream);
+                      int32_t *candidates, void *workspace, size_t workspace_bytes,
+                      void *stream);
 
 /*
  * Subsystem 4a — LRU lookup / touch / evict / slot-assign for one decode step.

@@ -226,13 +226,16 @@ def test_page_score_ordered_bounds_strided_query_view():
 
 
 # ------------------------------------------------------------------ top-k
-def run_topk(scores, rep, k):
+def run_topk(scores, rep, k, one_launch=False):
+    """one_launch: no candidate buffer, so rows longer than 16384 pages take the
+    single-workgroup walk instead of the two-launch selection."""
     from dram_attention_amd.topk_selector import topk_pages
 
     n_rows, H, L = scores.shape
     seq = n_rows // rep
     out = torch.empty(seq, H, rep, k, dtype=torch.int64, device=DEV)
-    topk_pages(scores.to(DEV), rep, k, out, H * rep * k, rep * k, k)
+    ws = torch.empty(0, dtype=torch.uint8, device=DEV) if one_launch else None
+    topk_pages(scores.to(DEV), rep, k, out, H * rep * k, rep * k, k, workspace=ws)
     return out.cpu()
 
 
@@ -241,12 +244,40 @@ def run_topk(scores, rep, k):
                                             (1, 1, 1, 1, 1), (2, 1, 2, 5000, 1),
                                             (8, 8, 2, 20000, 512), (1, 1, 1, 300, 299),
                                             (2, 1, 1, 65536, 8192), (8, 8, 1, 65536, 512),
-                                            (1, 1, 1, 16385, 600)])
+                                            (1, 1, 1, 16385, 600), (2, 2, 1, 16390, 8190),
+                                            (1, 1, 2, 300000, 64), (1, 1, 1, 40000, 30000)])
 def test_topk_pages_exact(rows, rep, H, L, k):
+    """Rows beyond 16384 pages go through the two-launch selection (parts, then
+    candidates) where the parts can each hold k pages, and through one workgroup
+    per row otherwise or without a candidate buffer: all against the stable sort."""
+    from dram_attention_amd import _lib
+
     scores = torch.randn(rows, H, L, generator=gen(13))
-    got = run_topk(scores, rep, k)
     want = O.select_pages(scores, rows // rep, rep, k)
-    assert same(got, want)
+    if k <= 8192:
+        assert same(run_topk(scores, rep, k), want)
+        assert same(run_topk(scores, rep, k, one_launch=True), want)
+    split = _lib.load().da_topk_pages_workspace_bytes(rows, H, L, k) > 0
+    assert split == ((rows, rep, H, L, k) in [(8, 8, 2, 20000, 512), (2, 1, 1, 65536, 8192),
+                                              (8, 8, 1, 65536, 512), (1, 1, 1, 16385, 600),
+                                              (2, 2, 1, 16390, 8190), (1, 1, 2, 300000, 64)])
+    if k > 8192:
+        with pytest.raises(RuntimeError, match="survivors"):
+            run_topk(scores, rep, k)
+
+
+def test_topk_pages_long_rows_with_ties_across_parts():
+    """Few distinct values over rows of 50 000 pages: the winners of equal score must be
+    the lowest page numbers whichever part they lie in, also when one part alone could
+    fill the list."""
+    scores = torch.randint(0, 3, (2, 2, 50000), generator=gen(17)).float()
+    scores[0, 0, 30000:] = 5.0          # one part holds more than k pages of the top value
+    scores[1, 1, :] = -2.0              # a constant row: pages 0..k-1
+    for k in (700, 8192):
+        want = torch.sort(scores, dim=-1, descending=True, stable=True).indices[..., :k]
+        got = run_topk(scores, 2, k)
+        assert same(got[0], want.transpose(0, 1)), k
+        assert same(run_topk(scores, 2, k, one_launch=True), got), k
 
 
 def test_topk_pages_bf16_rounded_scores_at_1m_row_length():
@@ -256,6 +287,44 @@ def test_topk_pages_bf16_rounded_scores_at_1m_row_length():
     got = run_topk(scores, 4, 512)
     want = torch.sort(scores, dim=-1, descending=True, stable=True).indices[..., :512]
     assert same(got[0], want.transpose(0, 1))
+
+
+@pytest.mark.parametrize("L,k", [(1000, 1000), (5000, 5000), (8192, 8192), (700, 513), (9000, 1025),
+                                 (16384, 4096), (3000, 2999), (64, 64), (1, 1)])
+@pytest.mark.parametrize("kind", ["normal", "rounded", "levels", "steps"])
+def test_topk_pages_long_lists_and_complete_orderings(L, k, kind):
+    """More than 512 winners are ordered by the stable radix sort of the survivors, and
+    k == L (a complete ordering) skips the selection: random fp32 scores (all four
+    digits differ), scores rounded to bf16 with both signs, a handful of levels (ties
+    by lowest page everywhere) and small whole numbers as the LRU's time stamps are."""
+    g = gen(100 + L + k)
+    if kind == "normal":
+        scores = torch.randn(2, 2, L, generator=g)
+    elif kind == "rounded":
+        scores = (torch.randn(2, 2, L, generator=g) * 8).bfloat16().float()
+    elif kind == "levels":
+        scores = torch.randint(-3, 4, (2, 2, L), generator=g).float()
+    else:
+        scores = -torch.randint(0, 300, (2, 2, L), generator=g).float()
+    want = torch.sort(scores, dim=-1, descending=True, stable=True).indices[..., :k]
+    assert same(run_topk(scores, 2, k)[0], want.transpose(0, 1))
+
+
+@pytest.mark.parametrize("ttype", [torch.float32, torch.int32])
+@pytest.mark.parametrize("N,kc", [(4096, 4096), (2048, 2048), (4096, 1500), (600, 600), (5000, 256)])
+def test_lru_candidates_are_the_stable_order_of_the_access_times(N, kc, ttype):
+    """The candidate list is the head of argsort(access_time, stable=True), up to the
+    complete order of all slots."""
+    from dram_attention_amd.lru_kernel import LruScratch, lru_candidates
+
+    H = 3
+    time = torch.randint(0, 900, (H, N), generator=gen(N + kc)).to(ttype)
+    time[1] = 7                                  # one head with every slot tied
+    sc = LruScratch.allocate(H, 16, DEV, N)._replace(
+        candidates=torch.empty(H, kc, dtype=torch.int32, device=DEV))
+    got = lru_candidates(time.to(DEV), sc).cpu().long()
+    want = torch.sort(time, dim=-1, stable=True).indices[:, :kc]
+    assert same(got, want)
 
 
 def test_empty_inputs_are_no_ops():
