@@ -108,17 +108,9 @@ inline SplitPlan plan_split(int64_t n_pages, int kp) {
 __global__ void __launch_bounds__(kSelThreads)
 topk_parts_kernel(const float *__restrict__ scores, int64_t row_stride, int64_t head_stride,
                   int n_rows, int n_pages, int kp, int n_parts, int part_len,
-                  uint32_t *__restrict__ cand_key, uint32_t *__restrict__ cand_page,
-                  const LruCandidateArgs cand) {
+                  uint32_t *__restrict__ cand_key, uint32_t *__restrict__ cand_page) {
   __shared__ SelectShared sm;
   const int h = blockIdx.y;
-  if ((int)blockIdx.x >= n_rows * n_parts) {
-    if (cand.time_is_i32)
-      lru_candidates_block<int32_t>(cand, h, sm);
-    else
-      lru_candidates_block<float>(cand, h, sm);
-    return;
-  }
   const int n = blockIdx.x / n_parts, part = blockIdx.x % n_parts;
   const int first = part * part_len;
   const int len = n_pages - first < part_len ? n_pages - first : part_len;
@@ -156,10 +148,21 @@ struct CandidateKey {
 template <typename IdxT>
 __global__ void __launch_bounds__(kSelThreads)
 topk_merge_kernel(const uint32_t *__restrict__ cand_key, const uint32_t *__restrict__ cand_page,
-                  int rep, int kp, int n_parts, IdxT *__restrict__ out, int64_t out_seq_stride,
-                  int64_t out_head_stride, int64_t out_rep_stride) {
+                  int n_rows, int rep, int kp, int n_parts, IdxT *__restrict__ out,
+                  int64_t out_seq_stride, int64_t out_head_stride, int64_t out_rep_stride,
+                  const LruCandidateArgs cand) {
   __shared__ SelectShared sm;
   const int n = blockIdx.x, h = blockIdx.y;
+  if (n >= n_rows) {
+    // The LRU candidates ride in this launch, the one with few workgroups: the
+    // parts of the 1M shape fill the device exactly (64 rows x 4 parts on 256
+    // compute units, one workgroup each), and eight more would run as a second round.
+    if (cand.time_is_i32)
+      lru_candidates_block<int32_t>(cand, h, sm);
+    else
+      lru_candidates_block<float>(cand, h, sm);
+    return;
+  }
   const int64_t base = ((int64_t)n * gridDim.y + h) * n_parts * kp;
   CandidateKey key{cand_key + base, (((uintptr_t)(cand_key + base)) & 15) == 0};
   const uint32_t *best = select_sorted(key, n_parts * kp, kp, sm);
@@ -222,18 +225,18 @@ extern "C" int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_
       (int64_t)rows * plan.n_parts < 0x7fffffff) {
     uint32_t *cand_key = (uint32_t *)workspace;
     uint32_t *cand_page = cand_key + (size_t)rows * n_heads * plan.row_words();
-    dim3 grid1(rows * plan.n_parts + (with_cand ? 1 : 0), n_heads), grid2(rows, n_heads);
+    dim3 grid1(rows * plan.n_parts, n_heads), grid2(rows + (with_cand ? 1 : 0), n_heads);
     hipLaunchKernelGGL(topk_parts_kernel, grid1, dim3(kSelThreads), 0, s, scores, row_stride,
                        head_stride, rows, (int)n_pages, kp, plan.n_parts, plan.part_len, cand_key,
-                       cand_page, cand);
+                       cand_page);
     if (out_itype == DA_I64)
       hipLaunchKernelGGL(topk_merge_kernel<int64_t>, grid2, dim3(kSelThreads), 0, s, cand_key,
-                         cand_page, rep, kp, plan.n_parts, (int64_t *)out, out_seq_stride,
-                         out_head_stride, out_rep_stride);
+                         cand_page, rows, rep, kp, plan.n_parts, (int64_t *)out, out_seq_stride,
+                         out_head_stride, out_rep_stride, cand);
     else
       hipLaunchKernelGGL(topk_merge_kernel<int32_t>, grid2, dim3(kSelThreads), 0, s, cand_key,
-                         cand_page, rep, kp, plan.n_parts, (int32_t *)out, out_seq_stride,
-                         out_head_stride, out_rep_stride);
+                         cand_page, rows, rep, kp, plan.n_parts, (int32_t *)out, out_seq_stride,
+                         out_head_stride, out_rep_stride, cand);
     return launch_status("da_topk_pages");
   }
   dim3 grid(rows + (with_cand ? 1 : 0), n_heads);

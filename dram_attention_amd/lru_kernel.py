@@ -93,6 +93,16 @@ def lru_update(
         _lib.require_gpu(t, name)
         if t.dim() > 1 and t.shape[-1] > 1 and t.stride(-1) != 1:
             raise ValueError(f"{name} must be dense along its last axis")
+    # the kernel indexes these by slot and by page: their extents must be the stores'
+    for name, t, want in (("page_access_time", page_access_time, (num_heads, num_hbm_pages)),
+                          ("hbm_page_to_dram_page_mapping", hbm_page_to_dram_page_mapping,
+                           (num_heads, num_hbm_pages)),
+                          ("dram_page_to_hbm_page_mapping", dram_page_to_hbm_page_mapping,
+                           (num_heads, num_dram_pages))):
+        if tuple(t.shape) != want:
+            raise ValueError(f"{name} has shape {tuple(t.shape)}, the page stores need {want}")
+    if topk_dram_page_index.shape[0] != num_heads:
+        raise ValueError("topk_dram_page_index must have one row per head")
     if dram_page_to_hbm_page_mapping.dtype != hbm_page_to_dram_page_mapping.dtype:
         raise TypeError("the two page mappings must share one integer type")
     if current_step.dtype != torch.int32:

@@ -556,6 +556,32 @@ def test_lru_update_forced_serial_walk_gives_the_same_state():
     lru_trace(2, 512, 128, 128, 6, 78, torch.int32, torch.int32, True, hot=64, serial_walk=True)
 
 
+def test_lru_update_rejects_maps_that_do_not_match_the_page_stores():
+    """The kernel indexes the access times and the slot->page map by slot and the
+    page->slot map by page: extents that differ from the stores' raise on the host,
+    before any launch."""
+    from dram_attention_amd.lru_kernel import LruScratch, lru_update
+
+    H, P, N, K = 2, 64, 8, 4
+    dram = torch.zeros(H, P, 16, device=DEV)
+    hbm = torch.zeros(H, N, 16, device=DEV)
+    good = dict(time=torch.zeros(H, N, device=DEV),
+                d2h=torch.full((H, P), -1, dtype=torch.int64, device=DEV),
+                h2d=torch.full((H, N), -1, dtype=torch.int64, device=DEV))
+    idx = torch.zeros(H, K, dtype=torch.int64, device=DEV)
+    step = torch.zeros(1, dtype=torch.int32, device=DEV)
+    sc = LruScratch.allocate(H, K, DEV, N)
+    for name, bad in (("time", torch.zeros(H, N - 1, device=DEV)),
+                      ("d2h", torch.full((H, P + 3), -1, dtype=torch.int64, device=DEV)),
+                      ("h2d", torch.full((H, 2 * N), -1, dtype=torch.int64, device=DEV))):
+        a = dict(good, **{name: bad})
+        with pytest.raises(ValueError, match="the page stores need"):
+            lru_update(dram, a["time"], a["d2h"], a["h2d"], idx, step, hbm, sc, True)
+    with pytest.raises(ValueError, match="one row per head"):
+        lru_update(dram, good["time"], good["d2h"], good["h2d"], idx[:1], step, hbm, sc, True)
+    assert step.item() == 0
+
+
 @pytest.mark.parametrize("H,P,N,K", [(2, 40, 6, 17), (1, 8, 2, 3), (3, 200, 50, 120),
                                      (2, 60, 10, 70)])
 def test_lru_update_more_requests_than_slots(H, P, N, K):
