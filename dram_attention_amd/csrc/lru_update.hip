@@ -127,9 +127,9 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       else
         atomic_min_signed(&d2h[p], (MapT)(kMarkerBase + k));  // smallest k wins
     }
-    if (t == 0) sm.n_miss = 0;
     __syncthreads();
     // -- phase B: rank the first occurrences in visiting order ---------------
+    uint32_t n_miss = 0;  // distinct misses so far (the same in every thread)
     for (int base = 0; base < K; base += kSelThreads) {
       const int k = base + t;
       bool first = false;
@@ -142,20 +142,14 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       const uint64_t m_first = __ballot(first);
       if (lane == 0) sm.wave_count[wave] = (uint32_t)__popcll(m_first);
       __syncthreads();
-      uint32_t before = sm.n_miss, round = 0;
-#pragma unroll
-      for (int w = 0; w < kSelWaves; ++w) {
-        const uint32_t c = sm.wave_count[w];
-        if (w < wave) before += c;
-        round += c;
-      }
+      uint32_t round;
+      const uint32_t before = n_miss + waves_prefix(sm.wave_count, round);
       const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
       if (first) sm.miss_page[before + (uint32_t)__popcll(m_first & below)] = (int32_t)p;
-      __syncthreads();
-      if (t == 0) sm.n_miss += round;
-      __syncthreads();
+      n_miss += round;
+      __syncthreads();  // miss_page is complete so far; wave_count may be rewritten
     }
-    const int m = (int)sm.n_miss;
+    const int m = (int)n_miss;
     // -- phase C: the m least recently used slots, in eviction order ---------
     const uint32_t *victims = nullptr;
     if (m > 0 && cand_all != nullptr && m <= k_cand) {
@@ -170,13 +164,8 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
         const uint64_t m_un = __ballot(untouched);
         if (lane == 0) sm.wave_count[wave] = (uint32_t)__popcll(m_un);
         __syncthreads();
-        uint32_t before = 0, total = 0;
-#pragma unroll
-        for (int w = 0; w < kSelWaves; ++w) {
-          const uint32_t c = sm.wave_count[w];
-          if (w < wave) before += c;
-          total += c;
-        }
+        uint32_t total;
+        const uint32_t before = waves_prefix(sm.wave_count, total);
         const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
         if (untouched)
           sm.sel.idx_out[kept + before + (uint32_t)__popcll(m_un & below)] = (uint32_t)slot;

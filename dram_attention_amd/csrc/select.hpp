@@ -50,7 +50,7 @@ struct alignas(16) SelectShared {
   alignas(16) uint32_t w32[kSelRankSortMax + 4];   // compact sort words
   uint32_t rank[kSelRankSortMax];
   uint32_t total[256];
-  uint32_t wave_gt[kSelWaves], wave_eq[kSelWaves];
+  uint32_t wave_pack[kSelWaves];  // per wave: (keys > T) << 16 | (keys == T)
   uint32_t low_or;       // OR over the normalised low 16 bits of all keys
   uint32_t digit;        // digit chosen by the current pass
   uint32_t remaining;    // how many keys are still wanted from the chosen bin
@@ -77,6 +77,19 @@ __device__ __forceinline__ uint32_t wave_scan_inclusive(uint32_t v) {
   v += dpp_u32<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
   v += dpp_u32<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
   return v;
+}
+
+// Exclusive prefix of this wave over the per-wave counts cnt[0..kSelWaves) in LDS,
+// and their total: lanes 0..15 take one count each, one more scan, and every wave
+// reads its own entry of the result (instead of a loop over the waves).  All 64
+// lanes of the calling wave must be active.
+__device__ __forceinline__ uint32_t waves_prefix(const uint32_t *cnt, uint32_t &total) {
+  const int lane = threadIdx.x & 63;
+  const uint32_t mine = lane < kSelWaves ? cnt[lane] : 0u;
+  const uint32_t upto = wave_scan_inclusive(mine);
+  const int my_wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  total = (uint32_t)__builtin_amdgcn_readlane((int)upto, kSelWaves - 1);
+  return (uint32_t)__builtin_amdgcn_readlane((int)(upto - mine), my_wave);
 }
 
 // Stable LSD radix sort of the words sel[0..k) by their key half (bits 63..32),
@@ -330,23 +343,16 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
       gt_c += kreg[u] > thresh ? 1u : 0u;
       eq_c += kreg[u] == thresh ? 1u : 0u;
     }
-    const uint32_t gt_incl = wave_scan_inclusive(gt_c), eq_incl = wave_scan_inclusive(eq_c);
-    if (lane == 63) {
-      sm.wave_gt[wave] = gt_incl;
-      sm.wave_eq[wave] = eq_incl;
-    }
+    // both counts in one word (a segment has at most 16384 keys: 15 bits each)
+    const uint32_t incl = wave_scan_inclusive((gt_c << 16) | eq_c);
+    if (lane == 63) sm.wave_pack[wave] = incl;
     __syncthreads();
-    uint32_t gt_off = gt_base + gt_incl - gt_c, eq_off = eq_base + eq_incl - eq_c;
-#pragma unroll
-    for (int w = 0; w < kSelWaves; ++w) {
-      const uint32_t g = sm.wave_gt[w], e = sm.wave_eq[w];
-      if (w < wave) {
-        gt_off += g;
-        eq_off += e;
-      }
-      gt_base += g;
-      eq_base += e;
-    }
+    uint32_t all;
+    const uint32_t before = waves_prefix(sm.wave_pack, all);
+    uint32_t gt_off = gt_base + (before >> 16) + (incl >> 16) - gt_c;
+    uint32_t eq_off = eq_base + (before & 0xffffu) + (incl & 0xffffu) - eq_c;
+    gt_base += all >> 16;
+    eq_base += all & 0xffffu;
     const int i0 = s * seg_n + t * C;
 #pragma unroll
     for (int u = 0; u < C; ++u) {
