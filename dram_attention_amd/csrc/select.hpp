@@ -385,6 +385,7 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
                           : 0u;
       __syncthreads();
       const uint32_t mine32 = ((uint32_t)(mine >> 32) & 0xffff0000u) | ((uint32_t)mine & 0xffffu);
+#pragma unroll 16
       for (int j = lo; j < hi; j += 4) {
         const uint4 v = *(const uint4 *)&sm.w32[j];  // padding words are 0: they beat nothing
         beat += (v.x > mine32) + (v.y > mine32) + (v.z > mine32) + (v.w > mine32);
