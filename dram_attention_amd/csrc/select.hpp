@@ -13,8 +13,9 @@
 //      in registers (16-byte loads); thread order is index order;
 //   2. MSB-first radix select, 8 bits per pass, finds the k-th largest key T.
 //      Histograms are replicated 32x so that clustered keys (rounded scores
-//      share their top digits) do not serialise the LDS atomics; if all keys
-//      agree in their low 16 bits (bf16-rounded scores) two passes suffice;
+//      share their top digits) do not serialise the LDS atomics; a digit in which
+//      no two keys differ needs no pass (scores rounded to bf16 differ in their
+//      high half only, time stamps of a decoding run in two digits at most);
 //   3. one block-wide scan of per-thread counts places every key > T and the
 //      lowest-index keys == T into LDS as 64-bit (key, ~index) words;
 //   4. the k survivors are ordered by rank counting (k <= 256: thread (e, slice)
@@ -51,7 +52,7 @@ struct alignas(16) SelectShared {
   uint32_t rank[kSelRankSortMax];
   uint32_t total[256];
   uint32_t wave_pack[kSelWaves];  // per wave: (keys > T) << 16 | (keys == T)
-  uint32_t low_or;       // OR over the normalised low 16 bits of all keys
+  uint32_t wave_or[kSelWaves], wave_nor[kSelWaves];  // per wave: OR over the (normalised) keys / their complements
   uint32_t digit;        // digit chosen by the current pass
   uint32_t remaining;    // how many keys are still wanted from the chosen bin
   uint32_t sort_or, sort_and;  // OR / AND over the keys of the survivors (radix sort)
@@ -76,6 +77,17 @@ __device__ __forceinline__ uint32_t wave_scan_inclusive(uint32_t v) {
   v += dpp_u32<0x118, 0xf>(v);  // row_shr:8  -> scan inside each 16-lane row
   v += dpp_u32<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
   v += dpp_u32<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+// OR over the 64 lanes of a wave, valid in lane 63 (the same DPP steps as the scan).
+__device__ __forceinline__ uint32_t wave_or_to_last_lane(uint32_t v) {
+  v |= dpp_u32<0x111, 0xf>(v);
+  v |= dpp_u32<0x112, 0xf>(v);
+  v |= dpp_u32<0x114, 0xf>(v);
+  v |= dpp_u32<0x118, 0xf>(v);
+  v |= dpp_u32<0x142, 0xa>(v);
+  v |= dpp_u32<0x143, 0xc>(v);
   return v;
 }
 
@@ -233,49 +245,70 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
   };
 
   const bool take_all = k == n;  // a complete ordering: nothing to select
-  // OR over the keys' low halves, complemented where the top bit is clear.  The
-  // order-preserving image of a float rounded to 16 bits ends in 0x0000 when its
-  // top bit is set and in 0xffff when it is clear (and the complemented image
-  // likewise): this OR is zero for such keys, and the high half alone orders them.
-  uint32_t low_or = 0;
+  // Which bits do two keys differ in?  OR over the keys and OR over their complements;
+  // a bit set in both is a 1 in one key and a 0 in another.  The low half is
+  // complemented first where the key's top bit is clear: the order-preserving image
+  // of a float rounded to 16 bits ends in 0x0000 when its top bit is set and in
+  // 0xffff when it is clear (and the complemented image likewise), so that such keys
+  // differ in their high half only, whatever their signs.
+  uint32_t acc_or = 0, acc_nor = 0;
   for (int s = n_seg - 1; s >= 0; --s) {  // ends with segment 0 in registers
     load_segment(s);
     const int real = n - (s * seg_n + t * C);
 #pragma unroll
-    for (int u = 0; u < C; ++u)
-      if (u < real)  // padding must not spoil the low-bits test
-        low_or |= kreg[u] ^ ~(uint32_t)((int32_t)kreg[u] >> 31);
+    for (int u = 0; u < C; ++u) {
+      if (u < real) {  // padding must not count
+        const uint32_t norm = kreg[u] ^ (~(uint32_t)((int32_t)kreg[u] >> 31) & 0xffffu);
+        acc_or |= norm;
+        acc_nor |= ~norm;
+      }
+    }
   }
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) low_or |= __shfl_xor(low_or, d, 64);
+  acc_or = wave_or_to_last_lane(acc_or);
+  acc_nor = wave_or_to_last_lane(acc_nor);
+  if (lane == 63) {
+    sm.wave_or[wave] = acc_or;
+    sm.wave_nor[wave] = acc_nor;
+  }
   for (int i = t; i < 256 * kHistCopies; i += kSelThreads) sm.hist[i] = 0;
   if (t < kSelRankSortMax) sm.rank[t] = 0;
   if (t == 0) {
     sm.remaining = (uint32_t)k;
-    sm.low_or = 0;
     sm.sort_or = 0;
     sm.sort_and = 0xffffffffu;
   }
   __syncthreads();
-  if (lane == 0 && (low_or & 0xffffu)) atomicOr(&sm.low_or, low_or & 0xffffu);
+  // every wave folds the 16 partial results for itself: no atomics, no second barrier
+  const uint32_t key_or = (uint32_t)__builtin_amdgcn_readlane(
+      (int)wave_or_to_last_lane(lane < kSelWaves ? sm.wave_or[lane] : 0u), 63);
+  const uint32_t key_nor = (uint32_t)__builtin_amdgcn_readlane(
+      (int)wave_or_to_last_lane(lane < kSelWaves ? sm.wave_nor[lane] : 0u), 63);
+  const uint32_t differ = key_or & key_nor;
 
   uint32_t prefix = 0;  // the digits of T fixed so far (high bits)
-  int passes = take_all ? 0 : 4;
+  const int passes = take_all ? 0 : 4;
+  bool counted = false;  // has a histogram pass run yet
   for (int pass = 0; pass < passes; ++pass) {
     const int shift = 24 - 8 * pass;
+    if (((differ >> shift) & 255u) == 0) {
+      // every key has the same digit here: it is the threshold's too (in the low
+      // half, undo the complement applied to keys whose top bit is clear)
+      uint32_t digit = (key_or >> shift) & 255u;
+      if (shift < 16 && !((prefix >> (23 - shift)) & 1u)) digit ^= 255u;
+      prefix = (prefix << 8) | digit;
+      continue;
+    }
     for (int s = 0; s < n_seg; ++s) {
       if (n_seg > 1) load_segment(s);
 #pragma unroll
       for (int u = 0; u < C; ++u) {
         const uint32_t key = kreg[u];
-        if (pass == 0 || (key >> (shift + 8)) == prefix)
+        if (!counted || (key >> (shift + 8)) == prefix)
           atomicAdd(&sm.hist[((key >> shift) & 255u) * kHistCopies + (lane & (kHistCopies - 1))], 1u);
       }
     }
+    counted = true;
     __syncthreads();
-    // every key's low half follows from its top bit (rounded scores, time stamps
-    // below 2^16 held as floats): the two low digits cannot separate anything
-    if (pass == 0 && sm.low_or == 0) passes = 2;
     if (t < 256) {
       uint32_t s = 0;
 #pragma unroll
@@ -318,8 +351,13 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     __syncthreads();
     prefix = (prefix << 8) | sm.digit;
   }
-  const bool low_const = passes == 2;
-  const uint32_t thresh = low_const ? (prefix << 16) | ((prefix >> 15) & 1 ? 0u : 0xffffu) : prefix;  // k-th largest key
+  const uint32_t thresh = prefix;  // k-th largest key
+  // Do the bits in which keys differ fit a window of 16?  (Rounded scores: the high
+  // half; time stamps of a run: a few low or middle bits.)  Then those bits order
+  // the keys: two keys that differ in their top bit put the window into the high
+  // half, where the complement of the low half plays no part.
+  const int key_lsb = differ ? __builtin_ctz(differ) : 16;
+  const bool narrow = (differ >> key_lsb) < 65536u && n <= 65536;
   const uint32_t n_eq = sm.remaining;  // keys == T to keep (k itself when nothing was selected)
   const uint32_t n_gt_total = (uint32_t)k - n_eq;
   // (the last barrier of the loop also retired every read of hist: sel may be written)
@@ -378,13 +416,13 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     const int hi = lo + per < k ? lo + per : k;
     const uint64_t mine = e < k ? sm.sel[e] : 0ull;
     uint32_t beat = 0;
-    if (low_const && n <= 65536) {
-      // key bits 31..16 and a 16-bit index say it all: 32-bit words
+    if (narrow) {
+      // the 16 key bits that can differ and a 16-bit index say it all: 32-bit words
       if (t < kSelRankSortMax + 4)
-        sm.w32[t] = t < k ? ((uint32_t)(sm.sel[t] >> 32) & 0xffff0000u) | ((uint32_t)sm.sel[t] & 0xffffu)
+        sm.w32[t] = t < k ? (((uint32_t)(sm.sel[t] >> 32) >> key_lsb) << 16) | ((uint32_t)sm.sel[t] & 0xffffu)
                           : 0u;
       __syncthreads();
-      const uint32_t mine32 = ((uint32_t)(mine >> 32) & 0xffff0000u) | ((uint32_t)mine & 0xffffu);
+      const uint32_t mine32 = (((uint32_t)(mine >> 32) >> key_lsb) << 16) | ((uint32_t)mine & 0xffffu);
 #pragma unroll 16
       for (int j = lo; j < hi; j += 4) {
         const uint4 v = *(const uint4 *)&sm.w32[j];  // padding words are 0: they beat nothing

@@ -310,6 +310,51 @@ def test_topk_pages_long_lists_and_complete_orderings(L, k, kind):
     assert same(run_topk(scores, 2, k)[0], want.transpose(0, 1))
 
 
+@pytest.mark.parametrize("k", [1, 37, 256, 700])
+@pytest.mark.parametrize("family", ["byte0", "byte1", "byte2", "byte3", "bytes12", "bits_10_21",
+                                    "signs_and_byte2", "signs_and_byte0", "rounded_both_signs",
+                                    "all_equal", "two_values"])
+def test_topk_pages_keys_that_differ_in_few_bits(family, k):
+    """The selection skips every digit in which no two keys differ and orders its winners on
+    the 16 bits that do when they fit a window: float scores built from bit patterns that
+    differ in one byte, in two, across a byte boundary, in the sign plus one byte, all
+    against the stable sort (values stay finite: exponent bits come from 0x3f.. or 0x40..)."""
+    g = gen(sum(map(ord, family)) + k)
+    L = 3000
+    r = lambda hi: torch.randint(0, hi, (2, 2, L), generator=g, dtype=torch.int64)
+    base = 0x40490000
+    bits = {
+        "byte0": base | r(256), "byte1": base | (r(256) << 8), "byte2": 0x40000000 | (r(128) << 16),
+        "byte3": (0x3f + r(3)) << 24 | 0x00400000, "bytes12": 0x40000000 | (r(65536) << 8) & 0x007fff00,
+        "bits_10_21": 0x40000000 | (r(4096) << 10),
+        "signs_and_byte2": (r(2) << 31) | 0x40000000 | (r(128) << 16),
+        "signs_and_byte0": (r(2) << 31) | base | r(256),
+        "rounded_both_signs": (r(2) << 31) | 0x3f000000 | (r(512) << 16),
+        "all_equal": torch.full((2, 2, L), base, dtype=torch.int64),
+        "two_values": base + 0x101 * r(2),
+    }[family]
+    scores = torch.from_numpy((bits & 0xffffffff).numpy().astype(np.uint32).view(np.float32))
+    assert torch.isfinite(scores).all()
+    want = torch.sort(scores, dim=-1, descending=True, stable=True).indices[..., :k]
+    assert same(run_topk(scores, 2, k)[0], want.transpose(0, 1))
+
+
+@pytest.mark.parametrize("ttype", [torch.float32, torch.int32])
+@pytest.mark.parametrize("lo,hi", [(0, 40), (4600, 5000), (60000, 70000), (16777000, 16777216),
+                                   (255, 258), (1000, 1001)])
+def test_lru_candidates_at_late_steps(lo, hi, ttype):
+    """Access times of a long decoding run (large step counts, a narrow window of them):
+    the short list of least recent slots is still the head of the stable order."""
+    from dram_attention_amd.lru_kernel import LruScratch, lru_candidates
+
+    H, N, kc = 2, 2048, 256
+    time = torch.randint(lo, hi, (H, N), generator=gen(lo + hi)).to(ttype)
+    sc = LruScratch.allocate(H, 16, DEV, N)._replace(
+        candidates=torch.empty(H, kc, dtype=torch.int32, device=DEV))
+    got = lru_candidates(time.to(DEV), sc).cpu().long()
+    assert same(got, torch.sort(time, dim=-1, stable=True).indices[:, :kc])
+
+
 @pytest.mark.parametrize("ttype", [torch.float32, torch.int32])
 @pytest.mark.parametrize("N,kc", [(4096, 4096), (2048, 2048), (4096, 1500), (600, 600), (5000, 256)])
 def test_lru_candidates_are_the_stable_order_of_the_access_times(N, kc, ttype):
