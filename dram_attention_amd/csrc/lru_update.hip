@@ -25,12 +25,16 @@ namespace da {
 
 constexpr int kLruMaxK = 8192;  // distinct-miss list kept in LDS (parallel path)
 
+constexpr int kLruTableMaxK = 4096;  // requests per head whose first misses are found in LDS
+
 struct LruShared {
   SelectShared sel;
   int32_t miss_page[kLruMaxK];
+  int16_t request_entry[kLruTableMaxK];  // per request: its entry of the page table, or kHit / kNoPage
   uint32_t wave_count[kSelWaves];
   uint32_t n_miss;
 };
+constexpr int16_t kHit = -1, kNoPage = -2;
 
 __device__ __forceinline__ void atomic_min_signed(int32_t *p, int32_t v) { atomicMin(p, v); }
 __device__ __forceinline__ void atomic_min_signed(int64_t *p, int64_t v) {
@@ -117,6 +121,69 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
     for (int i = t; i < m; i += kSelThreads)
       if (sm.miss_page[mslot[i]] != i) mslot[i] = -1;
   } else {
+    uint32_t n_miss = 0;  // distinct misses so far (the same in every thread)
+    const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    if (K <= kLruTableMaxK) {
+      // -- phases A and B through an LDS table --------------------------------
+      // A missed page goes into an open-addressing table in LDS (page -> lowest
+      // request position, twice as many entries as requests), and every request
+      // remembers its entry: the first occurrences are then found and ranked
+      // without another look at global memory.  The table borrows the selection
+      // area, which is idle until the victims are chosen.
+      int table_bits = 1;
+      while ((1 << table_bits) < 2 * K) ++table_bits;
+      const uint32_t mask = (1u << table_bits) - 1u;
+      int32_t *tab_page = (int32_t *)sm.sel.sel;  // 64 KiB: 2 x 8192 words at most
+      int32_t *tab_pos = tab_page + (mask + 1u);
+      for (uint32_t i = t; i <= mask; i += kSelThreads) {
+        tab_page[i] = -1;
+        tab_pos[i] = 0x7fffffff;
+      }
+      __syncthreads();
+      for (int k = t; k < K; k += kSelThreads) {
+        const int64_t p = (int64_t)idx[k];
+        int16_t entry = kNoPage;
+        if (p >= 0 && p < n_dram_pages) {
+          const int64_t s = (int64_t)d2h[p];
+          if (s >= 0) {
+            time[s] = now;
+            entry = kHit;
+          } else {
+            uint32_t e = ((uint32_t)p * 2654435761u) >> (32 - table_bits);
+            while (true) {
+              const int32_t old = atomicCAS(&tab_page[e], -1, (int32_t)p);
+              if (old == -1 || old == (int32_t)p) break;
+              e = (e + 1u) & mask;
+            }
+            atomicMin(&tab_pos[e], k);  // smallest k wins
+            entry = (int16_t)e;
+          }
+        }
+        sm.request_entry[k] = entry;
+      }
+      __syncthreads();
+      for (int base = 0; base < K; base += kSelThreads) {
+        const int k = base + t;
+        bool first = false;
+        int32_t p = -1;
+        if (k < K) {
+          const int16_t entry = sm.request_entry[k];
+          if (entry >= 0) {
+            first = tab_pos[entry] == k;
+            p = tab_page[entry];
+          }
+          if (hit) hit[k] = (entry != kNoPage && !first) ? 1 : 0;
+        }
+        const uint64_t m_first = __ballot(first);
+        if (lane == 0) sm.wave_count[wave] = (uint32_t)__popcll(m_first);
+        __syncthreads();
+        uint32_t round;
+        const uint32_t before = n_miss + waves_prefix(sm.wave_count, round);
+        if (first) sm.miss_page[before + (uint32_t)__popcll(m_first & below)] = p;
+        n_miss += round;
+        __syncthreads();  // miss_page is complete so far; wave_count may be rewritten
+      }
+    } else {
     // -- phase A: touch hits, mark the first occurrence of every missed page --
     for (int k = t; k < K; k += kSelThreads) {
       const int64_t p = (int64_t)idx[k];
@@ -129,7 +196,6 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
     }
     __syncthreads();
     // -- phase B: rank the first occurrences in visiting order ---------------
-    uint32_t n_miss = 0;  // distinct misses so far (the same in every thread)
     for (int base = 0; base < K; base += kSelThreads) {
       const int k = base + t;
       bool first = false;
@@ -144,10 +210,10 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       __syncthreads();
       uint32_t round;
       const uint32_t before = n_miss + waves_prefix(sm.wave_count, round);
-      const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
       if (first) sm.miss_page[before + (uint32_t)__popcll(m_first & below)] = (int32_t)p;
       n_miss += round;
       __syncthreads();  // miss_page is complete so far; wave_count may be rewritten
+    }
     }
     const int m = (int)n_miss;
     // -- phase C: the m least recently used slots, in eviction order ---------
