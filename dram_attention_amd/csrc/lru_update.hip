@@ -26,11 +26,14 @@ namespace da {
 constexpr int kLruMaxK = 8192;  // distinct-miss list kept in LDS (parallel path)
 
 constexpr int kLruTableMaxK = 4096;  // requests per head whose first misses are found in LDS
+constexpr int kLruBitmapSlots = 65536;  // slots per head whose hits are noted in LDS
+constexpr int32_t kNotFetched = -2;  // (a slot's old page was not requested ahead of time)
 
 struct LruShared {
   SelectShared sel;
   int32_t miss_page[kLruMaxK];
   int16_t request_entry[kLruTableMaxK];  // per request: its entry of the page table, or kHit / kNoPage
+  uint32_t touched[kLruBitmapSlots / 32];  // one bit per slot: hit in this step
   uint32_t wave_count[kSelWaves];
   uint32_t n_miss;
 };
@@ -123,6 +126,17 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
   } else {
     uint32_t n_miss = 0;  // distinct misses so far (the same in every thread)
     const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    // With the LDS table, hits are also noted in an LDS bitmap, and the head of the
+    // candidate list and the pages its slots hold are requested right away, long
+    // before the victims are chosen: choosing and re-mapping them then needs no
+    // further trip to global memory.
+    const bool use_bitmap = K <= kLruTableMaxK && n_hbm <= kLruBitmapSlots;
+    int32_t ahead_slot = -1, ahead_old = kNotFetched;
+    if (use_bitmap && cand_all != nullptr && t < k_cand) {
+      ahead_slot = cand_all[(int64_t)h * k_cand + t];
+      if (ahead_slot < 0 || ahead_slot >= n_hbm) ahead_slot = -1;  // not a slot: ignored
+      if (ahead_slot >= 0) ahead_old = (int32_t)h2d[ahead_slot];   // (page ids fit 32 bits)
+    }
     if (K <= kLruTableMaxK) {
       // -- phases A and B through an LDS table --------------------------------
       // A missed page goes into an open-addressing table in LDS (page -> lowest
@@ -139,6 +153,8 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
         tab_page[i] = -1;
         tab_pos[i] = 0x7fffffff;
       }
+      if (use_bitmap)
+        for (int i = t; i < (n_hbm + 31) / 32; i += kSelThreads) sm.touched[i] = 0;
       __syncthreads();
       for (int k = t; k < K; k += kSelThreads) {
         const int64_t p = (int64_t)idx[k];
@@ -147,6 +163,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
           const int64_t s = (int64_t)d2h[p];
           if (s >= 0) {
             time[s] = now;
+            if (use_bitmap) atomicOr(&sm.touched[s >> 5], 1u << (s & 31));
             entry = kHit;
           } else {
             uint32_t e = ((uint32_t)p * 2654435761u) >> (32 - table_bits);
@@ -223,23 +240,30 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       // touched anything: untouched slots keep their order and still precede every
       // touched one, so the first m untouched entries are the victims.
       uint32_t kept = 0;  // untouched entries found so far (the same in every thread)
+      int32_t *old_page = (int32_t *)sm.sel.sel;  // per victim: the page it held (the table is done with)
       for (int base = 0; base < k_cand && kept < (uint32_t)m; base += kSelThreads) {
         const int i = base + t;
-        const int32_t slot = i < k_cand ? cand_all[(int64_t)h * k_cand + i] : 0;
-        const bool untouched = i < k_cand && time[slot] != now;
+        const bool ahead = use_bitmap && base == 0;
+        int32_t slot = ahead ? ahead_slot : i < k_cand ? cand_all[(int64_t)h * k_cand + i] : -1;
+        if (slot >= n_hbm) slot = -1;
+        const bool untouched =
+            slot >= 0 && (use_bitmap ? !((sm.touched[slot >> 5] >> (slot & 31)) & 1u) : time[slot] != now);
         const uint64_t m_un = __ballot(untouched);
         if (lane == 0) sm.wave_count[wave] = (uint32_t)__popcll(m_un);
         __syncthreads();
         uint32_t total;
         const uint32_t before = waves_prefix(sm.wave_count, total);
-        const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-        if (untouched)
-          sm.sel.idx_out[kept + before + (uint32_t)__popcll(m_un & below)] = (uint32_t)slot;
+        if (untouched) {
+          const uint32_t at = kept + before + (uint32_t)__popcll(m_un & below);
+          sm.sel.idx_out[at] = (uint32_t)slot;
+          old_page[at] = ahead ? ahead_old : kNotFetched;
+        }
         kept += total;
         __syncthreads();  // idx_out is complete so far; wave_count may be rewritten
       }
       if (kept >= (uint32_t)m) victims = sm.sel.idx_out;  // else: too many were touched
     }
+    const bool have_old = victims != nullptr;
     if (m > 0 && victims == nullptr) {
       LeastRecentKey<TimeT> key{time};
       victims = select_sorted(key, n_hbm, m, sm.sel);
@@ -248,7 +272,8 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
     for (int i = t; i < m; i += kSelThreads) {
       const int32_t p = sm.miss_page[i];
       const int32_t v = (int32_t)victims[i];
-      const int64_t old = (int64_t)h2d[v];
+      const int32_t noted = have_old ? ((const int32_t *)sm.sel.sel)[i] : kNotFetched;
+      const int64_t old = noted != kNotFetched ? (int64_t)noted : (int64_t)h2d[v];
       if (old >= 0 && old < n_dram_pages) d2h[old] = (MapT)-1;
       h2d[v] = (MapT)p;
       d2h[p] = (MapT)v;
