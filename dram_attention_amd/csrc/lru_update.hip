@@ -70,8 +70,22 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
   int32_t *mslot = miss_slot_out + (int64_t)h * K;
   int32_t *slot_epoch = slot_epoch_all ? slot_epoch_all + (int64_t)h * n_hbm : nullptr;
 
-  const int32_t step = *step_ptr + (bump ? 1 : 0);
+  int32_t step_before = *step_ptr;
+  asm volatile("" : "+s"(step_before));  // the value has arrived: what follows cannot pass the read
+  const int32_t step = step_before + (bump ? 1 : 0);
   const TimeT now = (TimeT)step;
+  // The last head to have read the step publishes the bumped value and re-arms the
+  // ticket for the next call.  A head takes its ticket once its own read has
+  // returned, so whoever draws the last one knows that every read is done; the
+  // kernel boundary publishes the stores.  Taken here rather than at the end, the
+  // ticket's trip to memory is over long before the block is.
+  if (bump && t == 0) {
+    const int32_t done = atomicAdd(ticket, 1);
+    if (done == (int32_t)gridDim.x - 1) {
+      *step_ptr = step;
+      *ticket = 0;
+    }
+  }
 
   if (serial) {
     // -- literal restatement of the reference's three launches ---------------
@@ -285,17 +299,6 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
     if (t == 0) miss_count[h] = m;
   }
 
-  // The last head to finish publishes the bumped step and re-arms the ticket for
-  // the next call.  Every head has read the old value by then: its own ticket
-  // comes after that read in program order and depends on nothing another block
-  // wrote, so no fence is needed (the kernel boundary publishes the stores).
-  if (bump && t == 0) {
-    const int32_t done = atomicAdd(ticket, 1);
-    if (done == (int32_t)gridDim.x - 1) {
-      *step_ptr = step;
-      *ticket = 0;
-    }
-  }
 }
 
 // One 256-thread block per (entry, head), striding over the head's miss list.
