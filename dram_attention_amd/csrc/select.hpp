@@ -12,7 +12,7 @@
 //   1. a thread owns a CONTIGUOUS run of up to 16 indices and keeps those keys
 //      in registers (16-byte loads); thread order is index order;
 //   2. MSB-first radix select, 8 bits per pass, finds the k-th largest key T.
-//      Histograms are replicated 32x so that clustered keys (rounded scores
+//      Histograms are replicated 16x so that clustered keys (rounded scores
 //      share their top digits) do not serialise the LDS atomics; a digit in which
 //      no two keys differ needs no pass (scores rounded to bf16 differ in their
 //      high half only, time stamps of a decoding run in two digits at most);
@@ -35,7 +35,7 @@ namespace da {
 
 constexpr int kSelThreads = 1024;
 constexpr int kSelWaves = kSelThreads / 64;
-constexpr int kHistCopies = 32;
+constexpr int kHistCopies = 16;
 constexpr int kSelMaxK = 8192;     // survivors held in LDS: 8 bytes each
 constexpr int kSelRegKeys = 16;    // keys cached per thread
 constexpr int kSelRankSortMax = 256;  // longest list ordered by rank counting (measured: the
@@ -44,7 +44,7 @@ constexpr int kSelRankSortMax = 256;  // longest list ordered by rank counting (
 struct alignas(16) SelectShared {
   // the histogram phase and the survivor array never overlap in time
   union {
-    uint32_t hist[256 * kHistCopies];  // 32 KiB
+    uint32_t hist[256 * kHistCopies];  // 16 KiB
     uint64_t sel[kSelMaxK];            // 64 KiB
   };
   uint32_t idx_out[kSelMaxK];          // the result: winning indices, best first
