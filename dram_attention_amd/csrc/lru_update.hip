@@ -170,11 +170,28 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       if (use_bitmap)
         for (int i = t; i < (n_hbm + 31) / 32; i += kSelThreads) sm.touched[i] = 0;
       __syncthreads();
-      for (int k = t; k < K; k += kSelThreads) {
-        const int64_t p = (int64_t)idx[k];
+      // (the requests of all rounds are in flight together: two trips to memory for
+      // the phase, however many rounds of 1024 requests a head has)
+      constexpr int kRounds = kLruTableMaxK / kSelThreads;
+      int64_t page_of[kRounds], slot_of[kRounds];
+#pragma unroll
+      for (int r = 0; r < kRounds; ++r) {
+        const int k = r * kSelThreads + t;
+        page_of[r] = k < K ? (int64_t)idx[k] : -1;
+      }
+#pragma unroll
+      for (int r = 0; r < kRounds; ++r) {
+        if (page_of[r] >= n_dram_pages) page_of[r] = -1;
+        slot_of[r] = page_of[r] >= 0 ? (int64_t)d2h[page_of[r]] : -1;
+      }
+#pragma unroll
+      for (int r = 0; r < kRounds; ++r) {
+        const int k = r * kSelThreads + t;
+        if (k >= K) continue;
+        const int64_t p = page_of[r];
         int16_t entry = kNoPage;
-        if (p >= 0 && p < n_dram_pages) {
-          const int64_t s = (int64_t)d2h[p];
+        if (p >= 0) {
+          const int64_t s = slot_of[r];
           if (s >= 0) {
             time[s] = now;
             if (use_bitmap) atomicOr(&sm.touched[s >> 5], 1u << (s & 31));
