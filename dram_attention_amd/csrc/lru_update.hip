@@ -70,8 +70,9 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
   int32_t *mslot = miss_slot_out + (int64_t)h * K;
   int32_t *slot_epoch = slot_epoch_all ? slot_epoch_all + (int64_t)h * n_hbm : nullptr;
 
-  int32_t step_before = *step_ptr;
-  asm volatile("" : "+s"(step_before));  // the value has arrived: what follows cannot pass the read
+  int32_t step_read = *step_ptr;
+  asm volatile("" : "+v"(step_read)::"memory");  // the value has arrived: what follows cannot pass the read
+  const int32_t step_before = __builtin_amdgcn_readfirstlane(step_read);
   const int32_t step = step_before + (bump ? 1 : 0);
   const TimeT now = (TimeT)step;
   // The last head to have read the step publishes the bumped value and re-arms the
