@@ -11,10 +11,12 @@
 // Proof sketch: touched slots carry the largest time, so they sort behind the
 // M <= K - T victims consumed; a victim's old page is resident and untouched,
 // hence not among the requests, so no later request observes the eviction.
-// So the kernel does: touch hits and mark first occurrences of missed pages
-// (atomicMin of a position marker in the page->slot map), rank those
-// occurrences with a block scan, select the M least-recent slots in order
-// (select_sorted), and rewrite both maps in parallel.
+// So the kernel does: touch hits and find the first occurrence of every missed
+// page (an open-addressing table in LDS, page -> lowest request position; for
+// more than 4096 requests per head an atomicMin marker in the page->slot map),
+// rank those occurrences with ballots and a scan over the waves, take the M
+// least-recent untouched slots in order (from the caller's candidate list, or
+// select_sorted over all slots), and rewrite both maps in parallel.
 // K > N_hbm (victims may wrap onto pages touched in the same step) keeps the
 // reference's literal serial walk on one lane per head.
 //

@@ -190,7 +190,8 @@ int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_t head_stri
  *                  touches from that list instead of ordering all slots again (it
  *                  orders them itself whenever the list is too short); a list
  *                  that does not describe the current access times gives wrong
- *                  evictions.  NULL / k_cand = 0: no list.
+ *                  evictions (entries that are no slot number are ignored).
+ *                  NULL / k_cand = 0: no list.
  *   slot_epoch   : optional (Hkv, N_hbm) int32; a slot handed to a missed page
  *                  gets the step value, so a later kernel can tell which slots
  *                  the page stream of this step is (still) writing
