@@ -285,6 +285,70 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
       (int)wave_or_to_last_lane(lane < kSelWaves ? sm.wave_nor[lane] : 0u), 63);
   const uint32_t differ = key_or & key_nor;
 
+  // When the bits in which keys differ span at most 12 positions (scores rounded to
+  // bf16 within 16 binades, time stamps of a run), ONE pass over that window finds
+  // the threshold: 1024 bins x 4 copies, 2048 x 2 or 4096 x 1 in the same 16 KiB, the
+  // window's raw bits as the digit (outside the window all keys agree, up to the
+  // complement of the low half that follows the top bit).
+  const int d_lsb = differ ? __builtin_ctz(differ) : 0;
+  const int d_width = differ ? 32 - __builtin_clz(differ) - d_lsb : 0;
+  const bool one_pass = !take_all && differ != 0 && d_width <= 12;
+  uint32_t thresh;  // k-th largest key
+  if (one_pass) {
+    const int wbits = d_width <= 10 ? 10 : d_width;
+    const int wshift = d_lsb + wbits <= 32 ? d_lsb : 32 - wbits;
+    const uint32_t wmask = (1u << wbits) - 1u;
+    const int copy_bits = 12 - wbits;  // 4 copies, 2, or 1
+    for (int s = 0; s < n_seg; ++s) {
+      if (n_seg > 1) load_segment(s);
+#pragma unroll
+      for (int u = 0; u < C; ++u)
+        atomicAdd(&sm.hist[(((kreg[u] >> wshift) & wmask) << copy_bits) + (lane & ((1 << copy_bits) - 1))], 1u);
+    }
+    __syncthreads();
+    // thread t takes the t-th group of four words from the top: one bin (four
+    // copies), two bins (two copies each) or four bins, in descending order
+    const int group = kSelThreads - 1 - t;
+    const uint4 w = *(const uint4 *)&sm.hist[4 * group];
+    uint32_t c[4];  // counts of the group's bins, highest bin first; unused ones 0
+    if (wbits == 10) {
+      c[0] = w.x + w.y + w.z + w.w;
+      c[1] = c[2] = c[3] = 0;
+    } else if (wbits == 11) {
+      c[0] = w.z + w.w;
+      c[1] = w.x + w.y;
+      c[2] = c[3] = 0;
+    } else {
+      c[0] = w.w;
+      c[1] = w.z;
+      c[2] = w.y;
+      c[3] = w.x;
+    }
+    const uint32_t mine = c[0] + c[1] + c[2] + c[3];
+    const uint32_t incl = wave_scan_inclusive(mine);
+    if (lane == 63) sm.wave_pack[wave] = incl;
+    __syncthreads();
+    uint32_t all;
+    const uint32_t excl = waves_prefix(sm.wave_pack, all) + incl - mine;
+    const uint32_t want = (uint32_t)k;
+    if (excl < want && want <= excl + mine) {  // true in exactly one thread
+      uint32_t above = excl;
+      int j = 0;  // which bin of the group, from the top
+#pragma unroll
+      for (int x = 0; x < 3; ++x) {
+        if (j == x && above + c[x] < want) {
+          above += c[x];
+          j = x + 1;
+        }
+      }
+      sm.digit = (uint32_t)(((group + 1) << (wbits - 10)) - 1 - j);
+      sm.remaining = want - above;  // still needed from inside that bin
+    }
+    __syncthreads();
+    thresh = (key_or & ~(wmask << wshift)) | (sm.digit << wshift);
+    // low-half bits outside the window: undo the complement where the top bit is clear
+    if (!(thresh >> 31)) thresh ^= 0xffffu & ~(wmask << wshift);
+  } else {
   uint32_t prefix = 0;  // the digits of T fixed so far (high bits)
   const int passes = take_all ? 0 : 4;
   bool counted = false;  // has a histogram pass run yet
@@ -351,7 +415,8 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     __syncthreads();
     prefix = (prefix << 8) | sm.digit;
   }
-  const uint32_t thresh = prefix;  // k-th largest key
+  thresh = prefix;
+  }
   // Do the bits in which keys differ fit a window of 16?  (Rounded scores: the high
   // half; time stamps of a run: a few low or middle bits.)  Then those bits order
   // the keys: two keys that differ in their top bit put the window into the high

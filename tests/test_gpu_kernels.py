@@ -313,7 +313,8 @@ def test_topk_pages_long_lists_and_complete_orderings(L, k, kind):
 @pytest.mark.parametrize("k", [1, 37, 256, 700])
 @pytest.mark.parametrize("family", ["byte0", "byte1", "byte2", "byte3", "bytes12", "bits_10_21",
                                     "signs_and_byte2", "signs_and_byte0", "rounded_both_signs",
-                                    "all_equal", "two_values"])
+                                    "all_equal", "two_values", "bits_13_23", "sign_and_bits_20_22",
+                                    "negative_low_bits", "negative_bits_6_17"])
 def test_topk_pages_keys_that_differ_in_few_bits(family, k):
     """The selection skips every digit in which no two keys differ and orders its winners on
     the 16 bits that do when they fit a window: float scores built from bit patterns that
@@ -332,6 +333,10 @@ def test_topk_pages_keys_that_differ_in_few_bits(family, k):
         "rounded_both_signs": (r(2) << 31) | 0x3f000000 | (r(512) << 16),
         "all_equal": torch.full((2, 2, L), base, dtype=torch.int64),
         "two_values": base + 0x101 * r(2),
+        "bits_13_23": 0x40000000 | (r(2048) << 13),                       # one pass over 11 bits
+        "sign_and_bits_20_22": (r(2) << 31) | ((0x3f0 + r(8)) << 20),     # 12 bits up to the sign
+        "negative_low_bits": 0xC0490000 | (r(512) << 4),                  # complemented low half
+        "negative_bits_6_17": 0xC0400000 | (r(4096) << 6),                # window across both halves
     }[family]
     scores = torch.from_numpy((bits & 0xffffffff).numpy().astype(np.uint32).view(np.float32))
     assert torch.isfinite(scores).all()
