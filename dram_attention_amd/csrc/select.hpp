@@ -208,6 +208,23 @@ __device__ __forceinline__ void radix_sort_survivors(SelectShared &sm, int k) {
   }
 }
 
+// Where the result goes.  IntoLds: the winners' indices are left in sm.idx_out (best
+// first) behind a barrier, and select_sorted returns that array.  Direct<F>: every
+// winner is handed to f(rank, index) by one thread as soon as its rank is known,
+// without the trip through idx_out and its barrier (the return value is unused).
+struct IntoLds {
+  static constexpr bool kDirect = false;
+  __device__ __forceinline__ void operator()(uint32_t, uint32_t) const {}
+};
+template <typename F>
+struct Direct {
+  F f;
+  static constexpr bool kDirect = true;
+  __device__ __forceinline__ void operator()(uint32_t rank, uint32_t index) const { f(rank, index); }
+};
+template <typename F>
+__device__ __forceinline__ Direct<F> direct(F f) { return Direct<F>{f}; }
+
 // KeyFn provides
 //   uint32_t operator()(int i)            key of index i (0 <= i < n)
 //   void load4(int i, uint32_t *k)        keys of i..i+3 (i % 4 == 0, i+3 < n)
@@ -218,9 +235,9 @@ __device__ __forceinline__ void radix_sort_survivors(SelectShared &sm, int k) {
 // Slots past the end of the row are padded with key 0 (the smallest key) at
 // the highest indices: they can never displace a real key, so no phase needs a
 // validity test.  C = keys per thread per segment (4, 8 or 16).
-template <int C, typename KeyFn>
+template <int C, typename KeyFn, typename Emit>
 __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
-                                              SelectShared &sm) {
+                                              SelectShared &sm, const Emit &emit) {
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wave = t >> 6;
@@ -498,23 +515,33 @@ __device__ const uint32_t *select_sorted_impl(const KeyFn &key_of, int n, int k,
     }
     if (e < k && beat) atomicAdd(&sm.rank[e], beat);
     __syncthreads();
-    if (slice == 0 && e < k) sm.idx_out[sm.rank[e]] = 0xffffffffu - (uint32_t)mine;
-    __syncthreads();
+    if (slice == 0 && e < k) {
+      if constexpr (Emit::kDirect)
+        emit(sm.rank[e], 0xffffffffu - (uint32_t)mine);
+      else
+        sm.idx_out[sm.rank[e]] = 0xffffffffu - (uint32_t)mine;
+    }
+    if constexpr (!Emit::kDirect) __syncthreads();
     return sm.idx_out;
   }
 
   radix_sort_survivors(sm, k);
-  for (int j = t; j < k; j += kSelThreads) sm.idx_out[j] = 0xffffffffu - (uint32_t)sm.sel[j];
-  __syncthreads();
+  for (int j = t; j < k; j += kSelThreads) {
+    if constexpr (Emit::kDirect)
+      emit((uint32_t)j, 0xffffffffu - (uint32_t)sm.sel[j]);
+    else
+      sm.idx_out[j] = 0xffffffffu - (uint32_t)sm.sel[j];
+  }
+  if constexpr (!Emit::kDirect) __syncthreads();
   return sm.idx_out;
 }
 
-template <typename KeyFn>
+template <typename KeyFn, typename Emit = IntoLds>
 __device__ __forceinline__ const uint32_t *select_sorted(const KeyFn &key_of, int n, int k,
-                                                         SelectShared &sm) {
-  if (n <= 4 * kSelThreads) return select_sorted_impl<4>(key_of, n, k, sm);
-  if (n <= 8 * kSelThreads) return select_sorted_impl<8>(key_of, n, k, sm);
-  return select_sorted_impl<16>(key_of, n, k, sm);
+                                                         SelectShared &sm, const Emit &emit = Emit()) {
+  if (n <= 4 * kSelThreads) return select_sorted_impl<4>(key_of, n, k, sm, emit);
+  if (n <= 8 * kSelThreads) return select_sorted_impl<8>(key_of, n, k, sm, emit);
+  return select_sorted_impl<16>(key_of, n, k, sm, emit);
 }
 
 }  // namespace da

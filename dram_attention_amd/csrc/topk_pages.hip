@@ -43,9 +43,9 @@ template <typename TimeT>
 __device__ __forceinline__ void lru_candidates_block(const LruCandidateArgs &c, int h,
                                                      SelectShared &sm) {
   LeastRecentKey<TimeT> key{(const TimeT *)c.access_time + h * c.time_head_stride};
-  const uint32_t *order = select_sorted(key, c.n_slots, c.k_cand, sm);
   int32_t *dst = c.out + (int64_t)h * c.k_cand;
-  for (int j = threadIdx.x; j < c.k_cand; j += kSelThreads) dst[j] = (int32_t)order[j];
+  select_sorted(key, c.n_slots, c.k_cand, sm,
+                direct([=](uint32_t rank, uint32_t slot) { dst[rank] = (int32_t)slot; }));
 }
 
 template <typename IdxT>
@@ -66,9 +66,9 @@ topk_pages_kernel(const float *__restrict__ scores, int64_t row_stride, int64_t 
   }
   const float *row = scores + n * row_stride + h * head_stride;
   ScoreKey key{row, ((uintptr_t)row & 15) == 0};
-  const uint32_t *best = select_sorted(key, n_pages, kp, sm);
   IdxT *dst = out + (n / rep) * out_seq_stride + h * out_head_stride + (n % rep) * out_rep_stride;
-  for (int j = threadIdx.x; j < kp; j += kSelThreads) dst[j] = (IdxT)best[j];
+  select_sorted(key, n_pages, kp, sm,
+                direct([=](uint32_t rank, uint32_t page) { dst[rank] = (IdxT)page; }));
 }
 
 // Long rows in two launches.  A single workgroup keeps 16384 keys in registers
@@ -116,13 +116,11 @@ topk_parts_kernel(const float *__restrict__ scores, int64_t row_stride, int64_t 
   const int len = n_pages - first < part_len ? n_pages - first : part_len;
   const float *row = scores + n * row_stride + h * head_stride + first;
   ScoreKey key{row, ((uintptr_t)row & 15) == 0};
-  const uint32_t *best = select_sorted(key, len, kp, sm);
   const int64_t base = (((int64_t)n * gridDim.y + h) * n_parts + part) * kp;
-  for (int j = threadIdx.x; j < kp; j += kSelThreads) {
-    const uint32_t i = best[j];
-    cand_key[base + j] = key(i);
-    cand_page[base + j] = (uint32_t)first + i;
-  }
+  select_sorted(key, len, kp, sm, direct([=](uint32_t rank, uint32_t i) {
+                  cand_key[base + rank] = key(i);
+                  cand_page[base + rank] = (uint32_t)first + i;
+                }));
 }
 
 struct CandidateKey {
@@ -165,9 +163,10 @@ topk_merge_kernel(const uint32_t *__restrict__ cand_key, const uint32_t *__restr
   }
   const int64_t base = ((int64_t)n * gridDim.y + h) * n_parts * kp;
   CandidateKey key{cand_key + base, (((uintptr_t)(cand_key + base)) & 15) == 0};
-  const uint32_t *best = select_sorted(key, n_parts * kp, kp, sm);
   IdxT *dst = out + (n / rep) * out_seq_stride + h * out_head_stride + (n % rep) * out_rep_stride;
-  for (int j = threadIdx.x; j < kp; j += kSelThreads) dst[j] = (IdxT)cand_page[base + best[j]];
+  select_sorted(key, n_parts * kp, kp, sm, direct([=](uint32_t rank, uint32_t i) {
+                  dst[rank] = (IdxT)cand_page[base + i];
+                }));
 }
 
 }  // namespace da
