@@ -81,7 +81,8 @@ struct TileShared {
 // Prefix and local chunks only (the pass over the miss list stays with the
 // vector kernel).  kRows: query rows kept at the end (4, 8 or 16 >= rep).
 template <typename T, int kD, int kRows>
-__device__ __forceinline__ void attention_tile_block(const AttnArgs &a, const int block_x) {
+__device__ __forceinline__ void attention_tile_block(const AttnArgs &a, const int block_x,
+                                                     const int h) {
   using Ops = MatrixOps<T>;
   using Sh = TileShared<kD, kRows>;
   constexpr int kSteps = kD / 32;                 // MFMAs of the first product; K loads per lane
@@ -95,7 +96,6 @@ __device__ __forceinline__ void attention_tile_block(const AttnArgs &a, const in
   const int wave = threadIdx.x >> 6;
   const int g = lane >> 4;
   const int c = lane & 15;
-  const int h = blockIdx.y;
   const int chunk_id = a.chunk_base + block_x;
 
   const int kind = chunk_id < a.n_pchunks ? 0 : 1;
@@ -299,7 +299,7 @@ __device__ __forceinline__ void attention_tile_block(const AttnArgs &a, const in
 template <typename T, int kD, int kRows>
 __global__ void __launch_bounds__(kAttnThreads)
 decode_attention_tile_kernel(const AttnArgs a) {
-  attention_tile_block<T, kD, kRows>(a, blockIdx.x);
+  attention_tile_block<T, kD, kRows>(a, blockIdx.x, blockIdx.y);
 }
 
 }  // namespace da
