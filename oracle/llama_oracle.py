@@ -15,9 +15,13 @@ position 0, preserves norms, and makes q.k a function of the position difference
 only; the scaled frequencies against the three hand-computed cases of the rule;
 the SwiGLU width against the published Llama-3 widths (8B: 14336, 70B: 28672);
 RMSNorm against the formula on a vector whose answer is known in closed form.
+``greedy_generate`` (the evaluation driver's loop, evaluate.py:75-121) against a
+scripted model whose next token is a known function of the last one: the
+page-aligned prefill length, the forced prompt tokens, both stop rules and the
+returned slice are then fixed by hand.
 """
 import math
-from typing import Dict, Optional
+from typing import Dict, List, Optional
 
 import torch
 
@@ -132,3 +136,33 @@ class LlamaOracle:
                                  p + "feed_forward.w2.weight")
         h = rms_norm(h[:, -1:, :], self.w["norm.weight"], a.norm_eps)
         return self._linear(h, "output.weight").float()
+
+
+def greedy_generate(oracle: "LlamaOracle", prefix: List[int], suffix: List[int], max_gen_len: int,
+                    page_size: int, stop_tokens, special_start: int) -> List[int]:
+    """The evaluation driver's decoding loop on the CPU model
+    (evaluation/dram-attention/evaluate.py:75-121): the prefix cut to whole pages is
+    the prefill; from there on one token per call, where position p + 1 takes the
+    prompt's token if the prompt reaches that far and the argmax of the logits at p
+    otherwise; the loop ends after writing a stop token or a token of the special
+    range, and the result is what lies between the end of the prompt and the last
+    position fed to the model."""
+    prompt = list(prefix) + list(suffix)
+    total = min(oracle.a.max_seq_len, len(prompt) + max_gen_len)
+    seq = torch.full((total,), -1, dtype=torch.long)
+    seq[: len(prompt)] = torch.tensor(prompt, dtype=torch.long)
+    given = seq >= 0
+    start = len(prefix) // page_size * page_size
+    logits = oracle.forward(seq[None, :start], 0)
+    if not given[start]:
+        seq[start] = logits[0, -1].argmax()
+    last_fed = start
+    for p in range(start, total - 1):
+        last_fed = p
+        logits = oracle.forward(seq[None, p: p + 1], p)
+        if not given[p + 1]:
+            seq[p + 1] = logits[0, -1].argmax()
+        t = int(seq[p + 1])
+        if t in stop_tokens or t >= special_start:
+            break
+    return seq[len(prompt): last_fed + 1].tolist()

@@ -159,3 +159,69 @@ def test_model_variants_full_quest_and_quest_oracle():
     assert (outs["dram"] - outs["quest"]).abs().max().item() > 1e-4 * scale
     with pytest.raises(AssertionError):
         small_args(torch.float32, attention_variant="sparse")
+
+
+def test_recall_harness_on_a_checkpoint_directory(tmp_path):
+    """The evaluation driver end to end on a small random checkpoint written the way
+    the Llama-3 download lays it out (params.json + consolidated.00.pth): the loaded
+    model decodes the token sequence the CPU restatement of the driver decodes from
+    the same weights (page-aligned prefill of 992 of 1003 prefix tokens, 11 + 9 forced
+    prompt tokens, then free running), for the paged model and, against the restatement
+    with a cache that holds everything, for the full-attention variant; then two
+    generated key-value items through tokenizer, model, answer extraction and results
+    file."""
+    import json
+
+    from dram_attention_amd import LRUCache
+    from dram_attention_amd import evaluate as E
+
+    tok = E.ByteTokenizer()
+    params = dict(dim=256, n_layers=2, n_heads=8, n_kv_heads=2, vocab_size=tok.n_words,
+                  multiple_of=32, ffn_dim_multiplier=1.3, norm_eps=1e-5, rope_theta=500000.0,
+                  use_scaled_rope=True)
+    cache = dict(lru_hbm_cache_size=256, cache_top_k=128, cache_page_size=16,
+                 local_cache_size=128 + 64, max_output_length=64, max_seq_len=1100)
+    donor = build(L.ModelArgs(dtype=torch.float32, **params, **cache), 7)
+    (tmp_path / "params.json").write_text(json.dumps(params))
+    weights = {k: v.detach().cpu() for k, v in donor.named_parameters()}
+    weights["rope.freqs"] = torch.zeros(16)         # older checkpoints carry the rope table
+    torch.save(weights, tmp_path / "consolidated.00.pth")
+
+    g = torch.Generator().manual_seed(11)
+    prefix = torch.randint(0, 256, (1003,), generator=g).tolist()
+    suffix = torch.randint(0, 256, (9,), generator=g).tolist()
+    for variant, oracle_cache in (("dram", 256), ("full", 1100)):
+        model = E.load_model(str(tmp_path), 1100, variant=variant, top_k=128, page_size=16,
+                             local_attn_window=128, local_margin=64, lru_hbm_cache_size=256,
+                             max_output_length=64, dtype=torch.float32)
+        assert model.params.local_cache_size == 128 + 64 and model.params.cache_top_k == 128
+        for (name, p), (_, q) in zip(model.named_parameters(), donor.named_parameters()):
+            assert torch.equal(p, q), name
+        got = E.generate(model, prefix, suffix, 24, page_size=16, stop_tokens=tok.stop_tokens,
+                         special_start=tok.special_start)
+        args = L.ModelArgs(dtype=torch.float32, **params, **dict(cache, lru_hbm_cache_size=oracle_cache))
+        want = M.greedy_generate(M.LlamaOracle(args, donor.state_dict()), prefix, suffix, 24, 16,
+                                 tok.stop_tokens, tok.special_start)
+        assert got == want and 1 <= len(got) <= 23, (variant, got, want)
+        a = model.layers[0].attention.dram_attention
+        assert a.dram_kv_cache_size == 816 and isinstance(a.lru_cache, LRUCache) == (variant == "dram")
+
+    # the question line is ~100 byte tokens: they, the completion and the tokens behind the
+    # last whole page of the prefix all land in the local cache's room for new rows
+    model = E.load_model(str(tmp_path), 1100, top_k=128, page_size=16, local_attn_window=128,
+                         local_margin=64, lru_hbm_cache_size=256, max_output_length=192,
+                         dtype=torch.float32)
+    items = E.synthetic_niah(2, 14, seed=3)
+    path = tmp_path / E.results_file_name(1100, "smoke")
+    recall = E.evaluate_items(model, tok, items, page_size=16, results_path=str(path), max_gen_len=8)
+    rows = [json.loads(line) for line in path.read_text().splitlines()]
+    assert [r["index"] for r in rows] == [0, 1] and all(r["recall"] in (0, 1) for r in rows)
+    assert recall == sum(r["recall"] for r in rows) / 2
+    assert "1100 |" in E.report(str(tmp_path))
+    del weights["norm.weight"]
+    torch.save(weights, tmp_path / "consolidated.00.pth")
+    with pytest.raises(KeyError, match="norm.weight"):
+        E.load_model(str(tmp_path), 1100, dtype=torch.float32)
+    (tmp_path / "params.json").write_text(json.dumps(dict(params, hidden=3)))
+    with pytest.raises(ValueError, match="hidden"):
+        E.load_model(str(tmp_path), 1100)
