@@ -43,9 +43,11 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="128k", choices=sorted(WORKLOAD_INDEX))
     ap.add_argument("--eager", action="store_true", help="no HIP graph: launch from Python each step")
-    ap.add_argument("--steps-per-graph", type=int, default=8,
-                    help="decode steps captured into one HIP graph (the reference's example "
-                         "captures a whole model step, i.e. 32 attention layers, per graph)")
+    ap.add_argument("--steps-per-graph", type=int, default=32,
+                    help="decode steps captured into one HIP graph, at most 32 (the reference's "
+                         "example captures a whole model step, i.e. 32 attention layers, per graph); "
+                         "if --steps is not a multiple, the largest divisor of --steps between half "
+                         "of this and this is taken, else single-step graphs make up the rest")
     ap.add_argument("--no-overlap", action="store_true",
                     help="page stream and attention serialised on one stream")
     ap.add_argument("--force-lru", action="store_true",
@@ -712,6 +714,8 @@ def main():
         with torch.cuda.graph(graph):
             model_step()
         spg = max(1, min(args.steps_per_graph, args.steps, Layer.MAX_STEPS_PER_GRAPH))
+        if args.steps % spg:  # equal graphs where a near divisor exists
+            spg = next((d for d in range(spg, (spg + 1) // 2 - 1, -1) if args.steps % d == 0), spg)
         if spg > 1:
             graph_many = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph_many):
