@@ -159,6 +159,10 @@ __device__ __forceinline__ void unpack<BF16>(const u32x4 &v, float *f) {
 }
 
 __device__ __forceinline__ u32x4 load16(const void *p) { return *(const u32x4 *)p; }
+// The same load marked as streaming: the data will not be read again soon.
+__device__ __forceinline__ u32x4 load16_stream(const void *p) {
+  return __builtin_nontemporal_load((const u32x4 *)p);
+}
 __device__ __forceinline__ void store16(void *p, const u32x4 &v) { *(u32x4 *)p = v; }
 
 // Sum over groups of `width` adjacent lanes (width a power of two <= 64);
