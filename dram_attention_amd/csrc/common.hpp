@@ -164,6 +164,9 @@ __device__ __forceinline__ u32x4 load16_stream(const void *p) {
   return __builtin_nontemporal_load((const u32x4 *)p);
 }
 __device__ __forceinline__ void store16(void *p, const u32x4 &v) { *(u32x4 *)p = v; }
+__device__ __forceinline__ void store16_stream(void *p, const u32x4 &v) {
+  __builtin_nontemporal_store(v, (u32x4 *)p);
+}
 
 // Sum over groups of `width` adjacent lanes (width a power of two <= 64);
 // every lane of a group ends with the group's total.

@@ -108,7 +108,8 @@ __device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, c
 #pragma unroll
     for (int u = 0; u < kGatherMaxLoads; ++u) {
       const int j = u * kGatherThreads + tid;
-      if (j < g.page_vecs) store16(dst + (int64_t)j * 16, buf[u]);
+      // (streaming stores: a slot is next read a step later, behind the whole first pass)
+      if (j < g.page_vecs) store16_stream(dst + (int64_t)j * 16, buf[u]);
     }
 #pragma unroll
     for (int u = 0; u < kGatherMaxLoads; ++u) {
