@@ -100,7 +100,7 @@ __device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, c
 #pragma unroll
     for (int u = 0; u < kGatherMaxLoads; ++u) {
       const int j = u * kGatherThreads + tid;
-      buf[u] = load16(v >= 0 && j < g.page_vecs ? src + (int64_t)j * 16 : g.q);
+      buf[u] = load16_stream(v >= 0 && j < g.page_vecs ? src + (int64_t)j * 16 : g.q);
     }
   };
   auto settle = [&](const u32x4 *buf, char *dst) {
