@@ -35,8 +35,6 @@ decode_stream_attend_kernel(const AttnArgs a, const GatherAttendArgs g, const in
   }
 }
 
-// The same with the matrix-core form of the attention pass (one block takes all
-// query rows of a kv head, so the grid has no row dimension).
 // Whether the page stream of a launch is long enough to hide a first attention
 // pass that only n_core blocks per kv head compute, each walking every
 // n_core-th chunk.  The stream is bound by the host link (about 54 bytes/ns for
@@ -51,6 +49,8 @@ __device__ __forceinline__ bool stream_hides_few_blocks(int64_t stream_bytes, in
   return rounds * chunk_ns * 10 <= stream_ns * 7;
 }
 
+// The same with the matrix-core form of the attention pass (one block takes all
+// query rows of a kv head, so the grid has no row dimension).
 // One launch, two roles, blocks numbered in one dimension and dispatched in that
 // order: for every kv head its g_blocks blocks of the page stream and n_core
 // blocks of the first attention pass, then one block for every other chunk.
@@ -93,8 +93,8 @@ decode_stream_attend_tile_kernel(const AttnArgs a, const GatherAttendArgs g, con
     attention_tile_block<T, kLanes * 8, kRowsAttn>(a, first, h);
     return;
   }
-  // (streaming loads: the pass has time, and the merge and the next step's scorer
-  // find more of their data in the caches: 128K shape, 0.6 us per step)
+  // (streaming loads: the pass has time, and the next step's scorer finds its
+  // summaries still in the memory-side cache: 128K shape, 0.4 us per step)
   for (int c = first; c < n_chunks; c += n_core) {
     attention_tile_block<T, kLanes * 8, kRowsAttn, true>(a, c, h);
     __syncthreads();  // the block's LDS is used again
