@@ -808,9 +808,6 @@ def main():
                            "events, except lru_update, which changes its state and is one launch between "
                            "two events, so that its figure holds ~4 us of event and launch latency (a "
                            "kernel trace shows 6.3-6.6 us at the 128K shape)",
-        "kernels_us_note": "events around 8 back-to-back launches per kernel, except lru_update: it "
-                           "changes its own input, so it is one launch and ~4 us of launch latency "
-                           "sit inside its figure (its kernel time in the profiler is ~9 us)",
         "page_score_GBps": score_gbps,
         "page_stream": {"requests_per_step": requests, "distinct_misses_per_step": miss_per_step,
                         "h2d_bytes_per_step": miss_per_step * page_bytes,
