@@ -666,6 +666,16 @@ def model_decode(w, steps, seed, dev):
             "launch": "one HIP graph per token (32 layers)"}
 
 
+def steps_per_graph(steps: int, wanted: int, limit: int) -> int:
+    """How many decode steps one captured graph holds: `wanted`, capped by `limit` and by
+    the number of timed steps; if that does not divide `steps`, the largest divisor of
+    `steps` between half of it and it (equal graphs, no single-step graphs at the end)."""
+    spg = max(1, min(wanted, steps, limit))
+    if steps % spg:
+        spg = next((d for d in range(spg, (spg + 1) // 2 - 1, -1) if steps % d == 0), spg)
+    return spg
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -713,9 +723,7 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             model_step()
-        spg = max(1, min(args.steps_per_graph, args.steps, Layer.MAX_STEPS_PER_GRAPH))
-        if args.steps % spg:  # equal graphs where a near divisor exists
-            spg = next((d for d in range(spg, (spg + 1) // 2 - 1, -1) if args.steps % d == 0), spg)
+        spg = steps_per_graph(args.steps, args.steps_per_graph, Layer.MAX_STEPS_PER_GRAPH)
         if spg > 1:
             graph_many = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph_many):

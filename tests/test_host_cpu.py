@@ -173,3 +173,17 @@ def test_bench_cpu_baseline_is_independent_of_staged_steps():
     assert "64 decode steps" in res["sample"]
     assert res["cfg0"]["value"] > 0
     assert set(res["stage_ms_per_step"]) == {"score", "top_k", "lru", "attention"}
+
+
+def test_bench_steps_per_graph_choice():
+    """Equal graphs where the step count allows: 20 timed steps are one graph of 20,
+    64 two of 32, 50 two of 25; 33 has no divisor between 16 and 32 and keeps 32 (+ 1
+    single step); the limits hold."""
+    import bench
+
+    f = bench.steps_per_graph
+    assert [f(n, 32, 32) for n in (20, 64, 256, 50, 48, 100, 33, 7, 1)] == [20, 32, 32, 25, 24, 25, 32, 7, 1]
+    assert f(64, 8, 32) == 8 and f(20, 8, 32) == 5 and f(64, 100, 32) == 32 and f(5, 0, 32) == 1
+    for n in range(1, 200):
+        spg = f(n, 32, 32)
+        assert 1 <= spg <= min(n, 32) and (n % spg == 0 or spg == min(n, 32))
