@@ -372,6 +372,30 @@ def test_decode_parity_random_small_shapes(seed):
     run_parity(w, 100 + seed, w.steps, *tol[w.dtype])
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_decode_parity_random_mid_size_shapes(seed):
+    """Seeded sweep at sizes where the first attention pass has many chunks per kv head and
+    the page stream of a step is long against it: the launch that carries both then lets
+    a few workgroups per kv head walk the chunks (several rounds, a ragged last one),
+    with 1, 2, 4 and 8 kv heads, GQA widths up to 8, both head sizes and three page sizes."""
+    rng = np.random.default_rng(7000 + seed)
+    dtype = [torch.bfloat16, torch.float16][seed % 2]
+    n_kv = [8, 4, 2, 1][seed % 4]
+    rep = int(rng.choice([1, 2, 4, 8]))
+    head_dim = int(rng.choice([64, 128]))
+    page = int(rng.choice([8, 16, 32]))
+    n_slots = int(rng.integers(160, 420))
+    n_pages = int(rng.integers(3 * n_slots, 5 * n_slots))
+    kp = int(rng.integers(n_slots // 8, n_slots // 3)) // rep + 1
+    w = WORKLOADS["128k"].scaled(
+        dtype=dtype, n_q_heads=n_kv * rep, n_kv_heads=n_kv, head_dim=head_dim, page_size=page,
+        dram_tokens=n_pages * page, local_cache=int(rng.integers(4, 40)) * page,
+        lru_tokens=n_slots * page, top_k_tokens=kp * page, steps=3)
+    tol = {torch.float16: (4e-3, 1e-2), torch.bfloat16: (2e-2, 1e-2)}
+    rate = run_parity(w, 300 + seed, w.steps, *tol[w.dtype])
+    assert rate < 0.98          # the steps really paged
+
+
 @pytest.mark.parametrize("seed", range(32))
 def test_stream_variants_agree_on_random_small_shapes(seed):
     """Same workload through the three ways of running the page stream: inside the
