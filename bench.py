@@ -309,8 +309,7 @@ def time_kernels(layer, steps):
         idx = lru._topk_idx
         cand = lru._scratch_for(idx.shape[1]).candidates   # least recent slots, listed by the same launch
         timed("topk_pages", lambda: topk_pages(scores, w.rep, k, idx, w.rep * k, idx.shape[1], k,
-                                               lru=(lru.page_access_time, cand)))
-        lru._have_candidates = True
+                                               lru=(lru.page_access_time, cand, lru.current_step)))
         scratch = timed("lru_update", lambda: lru.update_(idx), repeat=1)   # mutates its state
         pk, pv = lru.views()
         c_len = int(layer.pos_dev.item()) - m.dram_kv_cache_size

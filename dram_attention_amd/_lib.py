@@ -58,7 +58,7 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_int64, c_int, c_int, c_int, c_int64, c_int, c_void_p, c_int64,
          c_int64, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p,
-         c_size_t, c_void_p],
+         c_void_p, c_size_t, c_void_p],
     ),
     "da_pages_gather": (
         c_int,
@@ -116,6 +116,8 @@ class PagedOverlap(ctypes.Structure):
         ("hbm_head_stride_bytes", c_int64),
         ("hbm_slot_stride_bytes", c_int64),
         ("miss_page", c_void_p),
+        ("link_gbps", c_float),
+        ("block_gbps", c_float),
     ]
 
 _lib = None

@@ -229,7 +229,8 @@ static void launch_split(AttnArgs a, int first_chunk, int n_launch, int n_kv_hea
 template <typename T>
 static int launch_attention(const AttnArgs &a, int dtype, int phase, int n_kv_heads, int lanes,
                             int head_dim, void *out, int64_t out_head_stride, float *lse_out,
-                            const GatherAttendArgs *stream_args, hipStream_t s) {
+                            const GatherAttendArgs *stream_args, float link_gbps, float block_gbps,
+                            hipStream_t s) {
 #define DA_ATTN_LAUNCH(tail, first, count)                                     \
   switch (lanes) {                                                             \
     case 4: launch_split<T, 4, tail>(a, first, count, n_kv_heads, s); break;   \
@@ -243,7 +244,7 @@ static int launch_attention(const AttnArgs &a, int dtype, int phase, int n_kv_he
                      0, s, a, mode, head_dim, (char *)out, out_head_stride, lse_out)
   if (phase & DA_PHASE_STREAM) {
     int rc = launch_stream_attend(a, *stream_args, dtype, lanes, a.n_pchunks + a.n_lchunks,
-                                  n_kv_heads, s);
+                                  n_kv_heads, link_gbps, block_gbps, s);
     if (rc) return rc;
   } else if (phase & DA_PHASE_FIRST) {
     DA_ATTN_LAUNCH(false, 0, a.n_pchunks + a.n_lchunks)
@@ -406,7 +407,12 @@ extern "C" int da_decode_attention_paged(
   hipStream_t s = (hipStream_t)stream;
   if (p.n_p + p.n_l == 0) return fail(DA_EINVAL, "da_decode_attention: no key/value rows at all");
   GatherAttendArgs g = {};
+  float link_gbps = 0.f, block_gbps = 0.f;
   if (phase & DA_PHASE_STREAM) {
+    DA_REQUIRE(overlap->link_gbps >= 0.f && overlap->block_gbps >= 0.f,
+               "da_decode_attention: negative rate in the overlap description");
+    link_gbps = overlap->link_gbps;
+    block_gbps = overlap->block_gbps;
     const int64_t page_vecs = (int64_t)overlap->page_size * 2 * lanes;
     if (lanes > 32 || a.rep > 8 || page_vecs > kGatherThreads * kGatherMaxLoads)
       return fail(DA_ENOTSUP,
@@ -445,13 +451,13 @@ extern "C" int da_decode_attention_paged(
   switch (dtype) {
     case DA_F32:
       return launch_attention<F32>(a, dtype, phase, n_kv_heads, lanes, head_dim, out,
-                                   out_head_stride, lse_out, &g, s);
+                                   out_head_stride, lse_out, &g, link_gbps, block_gbps, s);
     case DA_F16:
       return launch_attention<F16>(a, dtype, phase, n_kv_heads, lanes, head_dim, out,
-                                   out_head_stride, lse_out, &g, s);
+                                   out_head_stride, lse_out, &g, link_gbps, block_gbps, s);
     default:
       return launch_attention<BF16>(a, dtype, phase, n_kv_heads, lanes, head_dim, out,
-                                    out_head_stride, lse_out, &g, s);
+                                    out_head_stride, lse_out, &g, link_gbps, block_gbps, s);
   }
 }
 

@@ -57,7 +57,8 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
                   int64_t d2h_head_stride, MapT *h2d_all, int64_t h2d_head_stride,
                   uint8_t *hit_mask, int32_t *miss_page_out, int32_t *miss_slot_out,
                   int32_t *miss_count, int32_t *slot_epoch_all, int32_t *ticket, int serial,
-                  const int32_t *cand_all, int k_cand) {
+                  const int32_t *cand_all_in, int k_cand) {
+  const int32_t *cand_all = cand_all_in;
   __shared__ LruShared sm;
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -72,23 +73,35 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
   int32_t *mslot = miss_slot_out + (int64_t)h * K;
   int32_t *slot_epoch = slot_epoch_all ? slot_epoch_all + (int64_t)h * n_hbm : nullptr;
 
+  // Every wave reads the step for itself and waits for the value right here
+  // (and for the stamp of the candidate list, requested with it).
+  int32_t stamp_read = cand_all != nullptr ? cand_all[(int64_t)gridDim.x * k_cand + h] : 0;
   int32_t step_read = *step_ptr;
-  asm volatile("" : "+v"(step_read)::"memory");  // the value has arrived: what follows cannot pass the read
+  asm volatile("" : "+v"(step_read), "+v"(stamp_read)::"memory");  // the values have arrived: what follows cannot pass the reads
   const int32_t step_before = __builtin_amdgcn_readfirstlane(step_read);
+  // The list describes the access times as they were when the step counter read
+  // `stamp`; every update that bumps the counter changes them.  A list made at
+  // another step (or handed to a call that does not bump, whose stamps cannot tell
+  // two states apart) is ignored, and the kernel orders the slots itself.
+  if (!(bump && __builtin_amdgcn_readfirstlane(stamp_read) == step_before)) cand_all = nullptr;
   const int32_t step = step_before + (bump ? 1 : 0);
   const TimeT now = (TimeT)step;
   // The last head to have read the step publishes the bumped value and re-arms the
-  // ticket for the next call.  A head takes its ticket once its own read has
-  // returned, so whoever draws the last one knows that every read is done; the
-  // kernel boundary publishes the stores.  Taken here rather than at the end, the
-  // ticket's trip to memory is over long before the block is.
-  if (bump && t == 0) {
-    const int32_t done = atomicAdd(ticket, 1);
-    if (done == (int32_t)gridDim.x - 1) {
-      *step_ptr = step;
-      *ticket = 0;
+  // ticket for the next call.  A head is sixteen readers, one per wave, so it takes
+  // its ticket behind the first block barrier of its path: every wave of the block
+  // has waited for its own read before it arrives there, and whoever draws the last
+  // ticket knows that every read of every head is done; the kernel boundary publishes
+  // the stores.  Taken that early rather than at the end, the ticket's trip to memory
+  // is over long before the block is.
+  auto draw_ticket = [&]() {
+    if (bump && t == 0) {
+      const int32_t done = atomicAdd(ticket, 1);
+      if (done == (int32_t)gridDim.x - 1) {
+        *step_ptr = step;
+        *ticket = 0;
+      }
     }
-  }
+  };
 
   if (serial) {
     // -- literal restatement of the reference's three launches ---------------
@@ -99,6 +112,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       if (s >= 0) time[s] = now;
     }
     __syncthreads();
+    draw_ticket();
     LeastRecentKey<TimeT> key{time};
     const uint32_t *order = select_sorted(key, n_hbm, n_hbm, sm.sel);  // full stable order
     if (t == 0) {
@@ -173,6 +187,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
       if (use_bitmap)
         for (int i = t; i < (n_hbm + 31) / 32; i += kSelThreads) sm.touched[i] = 0;
       __syncthreads();
+      draw_ticket();
       // (the requests of all rounds are in flight together: two trips to memory for
       // the phase, however many rounds of 1024 requests a head has)
       constexpr int kRounds = kLruTableMaxK / kSelThreads;
@@ -246,6 +261,7 @@ lru_update_kernel(const IdxT *__restrict__ idx_all, int64_t idx_head_stride, int
         atomic_min_signed(&d2h[p], (MapT)(kMarkerBase + k));  // smallest k wins
     }
     __syncthreads();
+    draw_ticket();
     // -- phase B: rank the first occurrences in visiting order ---------------
     for (int base = 0; base < K; base += kSelThreads) {
       const int k = base + t;

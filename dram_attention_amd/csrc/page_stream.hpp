@@ -212,7 +212,10 @@ __device__ __forceinline__ void gather_attend_block(const GatherAttendArgs &g, c
 }
 
 // The page stream and the first attention pass as one launch (stream_attention.hip).
+// link_gbps / block_gbps: what a kernel's reads of the host store reach on this box,
+// and what one workgroup alone on its compute unit reads from HBM (0 = defaults).
 int launch_stream_attend(const AttnArgs &a, const GatherAttendArgs &g, int dtype, int lanes,
-                         int n_chunks, int n_kv_heads, hipStream_t s);
+                         int n_chunks, int n_kv_heads, float link_gbps, float block_gbps,
+                         hipStream_t s);
 
 }  // namespace da

@@ -179,6 +179,9 @@ __device__ __forceinline__ void radix_sort_survivors(SelectShared &sm, int k) {
           place[u] = seen + below;
           if (below == 0) row[digit] = seen + (uint32_t)__popcll(peers);
         }
+        // the next round's reads of the row come after this round's store (no
+        // instruction: it only forbids the compiler to move LDS accesses across)
+        __builtin_amdgcn_wave_barrier();
       }
     }
     __syncthreads();

@@ -37,16 +37,23 @@ decode_stream_attend_kernel(const AttnArgs a, const GatherAttendArgs g, const in
 
 // Whether the page stream of a launch is long enough to hide a first attention
 // pass that only n_core blocks per kv head compute, each walking every
-// n_core-th chunk.  The stream is bound by the host link (about 54 bytes/ns for
-// reads issued by a kernel); a block alone on its compute unit reads a chunk at
-// about 30 bytes/ns plus a microsecond of set-up; the pass should be over at 0.7
-// of the stream.
+// n_core-th chunk.  The stream is bound by the host link (link_bytes_per_us, the
+// rate of reads issued by a kernel on this box: the caller measures it); a block
+// alone on its compute unit reads a chunk at block_bytes_per_us plus a
+// microsecond of set-up; the pass should be over at 0.7 of the stream.  Only
+// time depends on the two rates, never a result: whoever computes a chunk
+// leaves the same partial.
+struct StreamRates {
+  float link_bytes_per_us, block_bytes_per_us;
+};
+constexpr float kDefaultLinkGBps = 54.f, kDefaultBlockGBps = 30.f;
 __device__ __forceinline__ bool stream_hides_few_blocks(int64_t stream_bytes, int64_t chunk_bytes,
-                                                        int n_chunks, int n_core) {
-  const int64_t stream_ns = stream_bytes / 54;
-  const int64_t chunk_ns = chunk_bytes / 30 + 1000;
-  const int64_t rounds = (n_chunks + n_core - 1) / n_core;
-  return rounds * chunk_ns * 10 <= stream_ns * 7;
+                                                        int n_chunks, int n_core,
+                                                        const StreamRates &r) {
+  const float stream_us = (float)stream_bytes / r.link_bytes_per_us;
+  const float chunk_us = (float)chunk_bytes / r.block_bytes_per_us + 1.0f;
+  const float rounds = (float)((n_chunks + n_core - 1) / n_core);
+  return rounds * chunk_us <= stream_us * 0.7f;
 }
 
 // The same with the matrix-core form of the attention pass (one block takes all
@@ -66,7 +73,7 @@ __device__ __forceinline__ bool stream_hides_few_blocks(int64_t stream_bytes, in
 template <typename T, int kLanes, int kRowsAttn, int kRowsGather>
 __global__ void __launch_bounds__(kAttnThreads)
 decode_stream_attend_tile_kernel(const AttnArgs a, const GatherAttendArgs g, const int g_blocks,
-                                 const int n_core, const int n_chunks) {
+                                 const int n_core, const int n_chunks, const StreamRates rates) {
   const int b = blockIdx.x;
   const int per_head = g_blocks + n_core;
   const int n_first = per_head * g.n_kv_heads;
@@ -78,7 +85,8 @@ decode_stream_attend_tile_kernel(const AttnArgs a, const GatherAttendArgs g, con
   int64_t missed = 0;
   for (int hh = 0; hh < g.n_kv_heads; ++hh) missed += g.miss_count[hh];
   const bool few = stream_hides_few_blocks(missed * g.page_vecs * 16,
-                                           (int64_t)a.chunk * kLanes * 16 * 2, n_chunks, n_core);
+                                           (int64_t)a.chunk * kLanes * 16 * 2, n_chunks, n_core,
+                                           rates);
   int h, first;
   if (b < n_first) {
     h = b / per_head;
@@ -103,7 +111,7 @@ decode_stream_attend_tile_kernel(const AttnArgs a, const GatherAttendArgs g, con
 
 template <typename T, int kLanes>
 static void launch_stream_attend(AttnArgs a, const GatherAttendArgs &g, int g_blocks, int n_chunks,
-                                 int n_kv_heads, hipStream_t s) {
+                                 int n_kv_heads, const StreamRates &rates, hipStream_t s) {
   a.chunk_base = 0;
   const int rep = a.rep;
   // (rows of 512 bytes stay with the vector pass here: both roles' LDS would not fit a block)
@@ -116,10 +124,10 @@ static void launch_stream_attend(AttnArgs a, const GatherAttendArgs &g, int g_bl
       const dim3 grid((g_blocks + n_chunks) * n_kv_heads, 1, 1);
       if (rep > 4)
         hipLaunchKernelGGL((decode_stream_attend_tile_kernel<T, kLanes, 8, 8>), grid,
-                           dim3(kAttnThreads), 0, s, a, g, g_blocks, n_core, n_chunks);
+                           dim3(kAttnThreads), 0, s, a, g, g_blocks, n_core, n_chunks, rates);
       else
         hipLaunchKernelGGL((decode_stream_attend_tile_kernel<T, kLanes, 4, 4>), grid,
-                           dim3(kAttnThreads), 0, s, a, g, g_blocks, n_core, n_chunks);
+                           dim3(kAttnThreads), 0, s, a, g, g_blocks, n_core, n_chunks, rates);
       return;
     }
   }
@@ -140,23 +148,28 @@ static void launch_stream_attend(AttnArgs a, const GatherAttendArgs &g, int g_bl
 
 template <typename T>
 static int dispatch_stream_attend(const AttnArgs &a, const GatherAttendArgs &g, int lanes,
-                                  int n_chunks, int n_kv_heads, hipStream_t s) {
+                                  int n_chunks, int n_kv_heads, const StreamRates &rates,
+                                  hipStream_t s) {
   switch (lanes) {
-    case 4: launch_stream_attend<T, 4>(a, g, a.gather_blocks, n_chunks, n_kv_heads, s); break;
-    case 8: launch_stream_attend<T, 8>(a, g, a.gather_blocks, n_chunks, n_kv_heads, s); break;
-    case 16: launch_stream_attend<T, 16>(a, g, a.gather_blocks, n_chunks, n_kv_heads, s); break;
-    case 32: launch_stream_attend<T, 32>(a, g, a.gather_blocks, n_chunks, n_kv_heads, s); break;
+    case 4: launch_stream_attend<T, 4>(a, g, a.gather_blocks, n_chunks, n_kv_heads, rates, s); break;
+    case 8: launch_stream_attend<T, 8>(a, g, a.gather_blocks, n_chunks, n_kv_heads, rates, s); break;
+    case 16: launch_stream_attend<T, 16>(a, g, a.gather_blocks, n_chunks, n_kv_heads, rates, s); break;
+    case 32: launch_stream_attend<T, 32>(a, g, a.gather_blocks, n_chunks, n_kv_heads, rates, s); break;
     default: return fail(DA_ENOTSUP, "page stream with attention: rows of %d bytes", lanes * 16);
   }
   return launch_status("da_decode_attention(page stream + first pass)");
 }
 
 int launch_stream_attend(const AttnArgs &a, const GatherAttendArgs &g, int dtype, int lanes,
-                         int n_chunks, int n_kv_heads, hipStream_t s) {
+                         int n_chunks, int n_kv_heads, float link_gbps, float block_gbps,
+                         hipStream_t s) {
+  // 1 GB/s = 1000 bytes per microsecond; 0 = the rates of the box this was tuned on
+  const StreamRates rates = {(link_gbps > 0.f ? link_gbps : kDefaultLinkGBps) * 1000.f,
+                             (block_gbps > 0.f ? block_gbps : kDefaultBlockGBps) * 1000.f};
   switch (dtype) {
-    case DA_F32: return dispatch_stream_attend<F32>(a, g, lanes, n_chunks, n_kv_heads, s);
-    case DA_F16: return dispatch_stream_attend<F16>(a, g, lanes, n_chunks, n_kv_heads, s);
-    default: return dispatch_stream_attend<BF16>(a, g, lanes, n_chunks, n_kv_heads, s);
+    case DA_F32: return dispatch_stream_attend<F32>(a, g, lanes, n_chunks, n_kv_heads, rates, s);
+    case DA_F16: return dispatch_stream_attend<F16>(a, g, lanes, n_chunks, n_kv_heads, rates, s);
+    default: return dispatch_stream_attend<BF16>(a, g, lanes, n_chunks, n_kv_heads, rates, s);
   }
 }
 

@@ -36,7 +36,9 @@ struct LruCandidateArgs {
   int64_t time_head_stride;
   int time_is_i32;
   int n_slots, k_cand;
-  int32_t *out;  // (Hkv, k_cand)
+  int32_t *out;  // (Hkv, k_cand) lists, then Hkv stamp words
+  const int32_t *step;  // the LRU step counter: its value now is the list's stamp
+  int n_heads;
 };
 
 template <typename TimeT>
@@ -44,6 +46,9 @@ __device__ __forceinline__ void lru_candidates_block(const LruCandidateArgs &c, 
                                                      SelectShared &sm) {
   LeastRecentKey<TimeT> key{(const TimeT *)c.access_time + h * c.time_head_stride};
   int32_t *dst = c.out + (int64_t)h * c.k_cand;
+  // The stamp says which state of the access times the list describes: the update
+  // that consumes the list compares it with the step it reads.
+  if (threadIdx.x == 0) c.out[(int64_t)c.n_heads * c.k_cand + h] = *c.step;
   select_sorted(key, c.n_slots, c.k_cand, sm,
                 direct([=](uint32_t rank, uint32_t slot) { dst[rank] = (int32_t)slot; }));
 }
@@ -183,8 +188,8 @@ extern "C" int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_
                                  void *out, int64_t out_seq_stride, int64_t out_head_stride,
                                  int64_t out_rep_stride, int out_itype, const void *access_time,
                                  int64_t time_head_stride, int time_type, int n_hbm_pages,
-                                 int k_cand, int32_t *candidates, void *workspace,
-                                 size_t workspace_bytes, void *stream) {
+                                 int k_cand, int32_t *candidates, const int32_t *step,
+                                 void *workspace, size_t workspace_bytes, void *stream) {
   using namespace da;
   DA_REQUIRE(n_rows >= 0 && n_heads >= 0 && n_pages >= 0 && kp >= 0 && rep >= 1,
              "da_topk_pages: bad geometry (rows %d heads %d pages %lld kp %d rep %d)", n_rows,
@@ -200,6 +205,9 @@ extern "C" int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_
                kSelMaxK);
     DA_REQUIRE(time_type == DA_TIME_F32 || time_type == DA_TIME_I32,
                "da_topk_pages_lru: bad access-time type");
+    DA_REQUIRE(step != nullptr, "da_topk_pages_lru: a candidate list needs the step counter");
+    cand.step = step;
+    cand.n_heads = n_heads;
     cand.access_time = access_time;
     cand.time_head_stride = time_head_stride;
     cand.time_is_i32 = time_type == DA_TIME_I32;
@@ -257,5 +265,5 @@ extern "C" int da_topk_pages(const float *scores, int64_t row_stride, int64_t he
                              size_t workspace_bytes, void *stream) {
   return da_topk_pages_lru(scores, row_stride, head_stride, n_rows, rep, n_heads, n_pages, kp, out,
                            out_seq_stride, out_head_stride, out_rep_stride, out_itype, nullptr, 0,
-                           DA_TIME_F32, 0, 0, nullptr, workspace, workspace_bytes, stream);
+                           DA_TIME_F32, 0, 0, nullptr, nullptr, workspace, workspace_bytes, stream);
 }

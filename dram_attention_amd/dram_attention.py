@@ -17,7 +17,7 @@ import torch.nn.functional as F
 
 from . import _lib
 from .lru_cache import DummyCache, LRUCache
-from .lru_kernel import GATHER_BLOCKS, gather_attend_supported
+from .lru_kernel import GATHER_BLOCKS, gather_attend_supported, host_link_gbps
 from .topk_selector import TokenMaxTopKSelector
 
 
@@ -36,7 +36,8 @@ class PagedPrefix:
     FIRST, SECOND, FIRST_MERGE, STREAM, MERGE_ALL = 1, 2, 4, 8, 16
 
     def __init__(self, page_size: int, scratch, current_step: torch.Tensor, phase: int,
-                 gather_blocks: int = 0, page_stores=None):
+                 gather_blocks: int = 0, page_stores=None, link_gbps: float = 0.0,
+                 block_gbps: float = 0.0):
         self.page_size = page_size
         self.scratch = scratch
         self.current_step = current_step
@@ -47,6 +48,11 @@ class PagedPrefix:
         # STREAM: (dram_kv_cache, its device-visible address, hbm_kv_cache); the page
         # stream then runs inside the launch of the FIRST pass
         self.page_stores = page_stores
+        # STREAM: the host link's rate for reads issued by a kernel and the rate at which
+        # one workgroup reads HBM, GB/s (0 = the library's defaults); they decide how
+        # many workgroups compute the first pass next to a long stream, not what it computes
+        self.link_gbps = link_gbps
+        self.block_gbps = block_gbps
 
     def as_struct(self) -> "_lib.PagedOverlap":
         s = self.scratch
@@ -63,6 +69,7 @@ class PagedPrefix:
             o.dram_page_stride_bytes = dram.stride(1) * esz
             o.hbm_head_stride_bytes = hbm.stride(0) * esz
             o.hbm_slot_stride_bytes = hbm.stride(1) * esz
+            o.link_gbps, o.block_gbps = self.link_gbps, self.block_gbps
         return o
 
 
@@ -236,6 +243,14 @@ class DRAMAttention(torch.nn.Module):
         # of page selection (evaluation/quest-top-k-oracle/model.py:267-275); keeps all
         # prefix keys on the device.  Read by init_cache.
         self.page_selector = "bound"
+        # Workgroups of the page stream in all, and two rates of the machine (GB/s) that
+        # time the stream + attention launch: what a kernel's reads of the pinned store
+        # reach (set by init_cache from one timed pinned copy; a kernel gets about 0.95
+        # of a copy engine's rate) and what one workgroup alone reads from HBM (0 = the
+        # library's default).  Results do not depend on any of the three.
+        self.stream_blocks = GATHER_BLOCKS
+        self.link_gbps = 0.0
+        self.block_gbps = 0.0
 
     def init_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor):
         """Split the prompt's (1,S,Hkv,D) keys/values into the paged prefix and the
@@ -258,6 +273,7 @@ class DRAMAttention(torch.nn.Module):
                 lru_hbm_cache_size=self.lru_hbm_cache_size,
                 device=self.device,
             )
+            self.link_gbps = 0.95 * host_link_gbps(self.cache_k.device)
             if self.page_selector == "token_max":
                 self.lru_cache.top_k_selector = TokenMaxTopKSelector(
                     prefix_k, self.lru_cache.num_dram_pages, device=self.device)
@@ -388,7 +404,7 @@ class DRAMAttention(torch.nn.Module):
         # the shape allows; otherwise a tail pass covers them after the stream.
         fused = self.attend_on_page_stream and gather_attend_supported(
             Hq, self.n_kv_heads, D, self.page_size, xq.dtype)
-        blocks = max(1, min(GATHER_BLOCKS // self.n_kv_heads, k)) if fused else 0
+        blocks = max(1, min(self.stream_blocks // self.n_kv_heads, k)) if fused else 0
 
         def stream_pages():
             if fused:
@@ -416,7 +432,8 @@ class DRAMAttention(torch.nn.Module):
                 decode_attention(*args, workspace=self._workspace, out=out[0, 0],
                                  cache_len_offset=offset,
                                  paged=PagedPrefix(self.page_size, scratch, lru.current_step,
-                                                   phase, blocks, lru.page_stores()))
+                                                   phase, blocks, lru.page_stores(),
+                                                   self.link_gbps, self.block_gbps))
 
             if defer_merge:
                 launch(P.STREAM | P.FIRST)

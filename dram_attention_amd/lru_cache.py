@@ -136,7 +136,6 @@ class LRUCache(torch.nn.Module):
 
         self._scratch = None
         self._topk_idx = None
-        self._have_candidates = False
 
     # -- internals ---------------------------------------------------------
     def _scratch_for(self, k: int) -> LruScratch:
@@ -144,15 +143,6 @@ class LRUCache(torch.nn.Module):
             self._scratch = LruScratch.allocate(self.num_kv_heads, k, self.hbm_kv_cache.device,
                                                 self.num_hbm_pages)
         return self._scratch
-
-    def _candidates_fit(self, idx: torch.Tensor) -> bool:
-        """Whether the list of least recently used slots that select_ left is current for
-        an update with ``idx``: it is for the request list select_ itself produced, once,
-        provided nothing updated the cache in between."""
-        use = (self._have_candidates and self._topk_idx is not None
-               and idx.data_ptr() == self._topk_idx.data_ptr() and idx.shape == self._topk_idx.shape)
-        self._have_candidates = False
-        return use
 
     def _views(self) -> CacheOutput:
         paged = self.hbm_kv_cache.view(
@@ -172,7 +162,7 @@ class LRUCache(torch.nn.Module):
             self.dram_kv_cache, self.page_access_time, self.dram_page_to_hbm_page_mapping,
             self.hbm_page_to_dram_page_mapping, top_k_dram_page_index, self.current_step,
             self.hbm_kv_cache, scratch, bump_step=True, dram_device_ptr=self._dram_device_ptr,
-            use_candidates=self._candidates_fit(top_k_dram_page_index),
+            use_candidates=True,   # the kernel ignores a list whose stamp is not this step
         )
         return self._views()
 
@@ -199,17 +189,17 @@ class LRUCache(torch.nn.Module):
         # the same launch lists the least recently used slots for update_ (the
         # order of the slots does not depend on the scores)
         scratch = self._scratch_for(total)
-        self._have_candidates = True
         return self.top_k_selector.top_k_for_lru(
-            q, k, out=self._topk_idx, lru=(self.page_access_time, scratch.candidates))
+            q, k, out=self._topk_idx, lru=(self.page_access_time, scratch.candidates, self.current_step))
 
     def update_(self, idx: torch.Tensor) -> LruScratch:
         """Metadata only: advance the step, touch/evict/assign, emit the miss list."""
         scratch = self._scratch_for(idx.shape[1])
-        use = self._candidates_fit(idx)
+        # the list select_ left carries the step it was made at: the kernel uses it only
+        # if nothing has updated the cache since
         lru_update(self.dram_kv_cache, self.page_access_time, self.dram_page_to_hbm_page_mapping,
                    self.hbm_page_to_dram_page_mapping, idx, self.current_step, self.hbm_kv_cache,
-                   scratch, bump_step=True, use_candidates=use)
+                   scratch, bump_step=True, use_candidates=True)
         return scratch
 
     def gather_(self, k: int) -> None:

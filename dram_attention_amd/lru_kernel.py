@@ -22,7 +22,9 @@ class LruScratch(NamedTuple):
     hit_mask: torch.Tensor    # (H, K) uint8: 1 = resident when visited
     workspace: torch.Tensor   # zeroed once; holds the step-bump ticket
     slot_epoch: torch.Tensor  # (H, N_hbm) int32: step at which a slot was last re-assigned
-    candidates: torch.Tensor = None   # (H, k_cand) int32: least recent slots, when a selector fills it
+    # (H, k_cand) int32: least recent slots, when a selector fills it; a view made by
+    # candidate_list(), whose buffer carries one stamp word per head behind the lists
+    candidates: torch.Tensor = None
 
     @staticmethod
     def allocate(num_heads: int, k: int, device, num_hbm_pages: int = 0) -> "LruScratch":
@@ -36,9 +38,27 @@ class LruScratch(NamedTuple):
             miss_count=torch.zeros(num_heads, dtype=torch.int32, device=device),
             hit_mask=torch.empty(num_heads, max(k, 1), dtype=torch.uint8, device=device),
             workspace=torch.zeros(ws, dtype=torch.uint8, device=device),
-            candidates=torch.empty(num_heads, max(lru_candidate_count(k, num_hbm_pages), 1),
-                                   dtype=torch.int32, device=device),
+            candidates=candidate_list(num_heads, max(lru_candidate_count(k, num_hbm_pages), 1),
+                                      device),
         )
+
+
+def candidate_list(num_heads: int, k_cand: int, device) -> torch.Tensor:
+    """Room for the lists of least recently used slots as da_topk_pages_lru writes them:
+    an (H, k_cand) int32 view of a buffer that holds one stamp word per head behind the
+    lists (the step counter's value when a list was made; da_lru_update ignores a list
+    whose stamp is not the step it reads).  Starts out with stamps no counter has."""
+    buf = torch.full((num_heads * k_cand + num_heads,), -1, dtype=torch.int32, device=device)
+    return buf[: num_heads * k_cand].view(num_heads, k_cand)
+
+
+def check_candidate_list(candidates: torch.Tensor) -> None:
+    H, k_cand = candidates.shape
+    room = candidates.untyped_storage().nbytes() // 4 - candidates.storage_offset()
+    if (candidates.dtype != torch.int32 or not candidates.is_contiguous()
+            or room < H * k_cand + H):
+        raise ValueError("the candidate list must come from candidate_list(): contiguous int32 "
+                         "lists with one stamp word per head behind them")
 
 
 MIN_LRU_CANDIDATES = 256   # one sort block's fast path
@@ -75,7 +95,8 @@ def lru_update(
     ``scratch`` (one launch on the current stream).  ``serial_walk`` forces the
     literal one-request-at-a-time walk (same result, for checks and baselines).
     ``use_candidates``: ``scratch.candidates`` holds the least recently used slots
-    in eviction order as of right now (filled by ``topk_pages(..., lru=...)``)."""
+    in eviction order (filled by ``topk_pages(..., lru=...)``); the kernel uses the
+    list only if its stamp is the step it reads, i.e. if no update came in between."""
     num_heads, num_dram_pages, page_dim = dram_kv_cache.shape
     _, k = topk_dram_page_index.shape
     assert (
@@ -112,6 +133,8 @@ def lru_update(
     if dram_kv_cache.stride(2) != 1 or hbm_kv_cache.stride(2) != 1:
         raise ValueError("pages must be dense")
     epoch = scratch.slot_epoch if scratch.slot_epoch.shape == (num_heads, num_hbm_pages) else None
+    if use_candidates:
+        check_candidate_list(scratch.candidates)
     lib = _lib.load()
     _lib.check(
         lib.da_lru_update(
@@ -135,18 +158,22 @@ def lru_update(
     )
 
 
-def lru_candidates(page_access_time: torch.Tensor, scratch: LruScratch) -> torch.Tensor:
+def lru_candidates(page_access_time: torch.Tensor, scratch: LruScratch,
+                   current_step: torch.Tensor) -> torch.Tensor:
     """Fill ``scratch.candidates`` with the least recently used slots of every head, in
-    eviction order, as of now (one launch; normally this rides along with the top-k)."""
+    eviction order, as of now, stamped with ``current_step`` (one launch; normally this
+    rides along with the top-k)."""
     H, N = page_access_time.shape
     cand = scratch.candidates
     _lib.require_gpu(page_access_time, "page_access_time")
+    _lib.require_gpu(current_step, "current_step")
+    check_candidate_list(cand)
     _lib.check(
         _lib.load().da_topk_pages_lru(
             None, 0, 0, 0, 1, H, 0, 0, None, 0, 0, 0, _lib.itype_code(torch.int64),
             page_access_time.data_ptr(), page_access_time.stride(0),
-            _lib.time_code(page_access_time.dtype), N, cand.shape[1], cand.data_ptr(), None, 0,
-            _lib.stream_ptr(page_access_time.device)),
+            _lib.time_code(page_access_time.dtype), N, cand.shape[1], cand.data_ptr(),
+            current_step.data_ptr(), None, 0, _lib.stream_ptr(page_access_time.device)),
         "da_topk_pages_lru")
     return cand
 
@@ -173,6 +200,30 @@ def pages_gather(dram_kv_cache: torch.Tensor, hbm_kv_cache: torch.Tensor, scratc
 
 
 GATHER_BLOCKS = 32  # workgroups of a page stream in all: few and fat saturate the host link
+
+_link_gbps = {}
+
+
+def host_link_gbps(device) -> float:
+    """Pinned host -> HBM copy rate of this box in GB/s, measured once per device and
+    process (three 16 MiB copies between two events, under a millisecond).  Only the
+    scheduling of the stream + attention launch reads it, never a result."""
+    device = torch.device(device)
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    if key not in _link_gbps:
+        n = 16 << 20
+        src = torch.empty(n, dtype=torch.uint8, pin_memory=True)
+        dst = torch.empty(n, dtype=torch.uint8, device=device)
+        dst.copy_(src, non_blocking=True)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(3):
+            dst.copy_(src, non_blocking=True)
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_time(e1)
+        _link_gbps[key] = 3 * n / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+    return _link_gbps[key]
 
 
 def gather_attend_supported(n_q_heads: int, n_kv_heads: int, head_dim: int, page_size: int,

@@ -56,9 +56,10 @@ def topk_pages(scores: torch.Tensor, rep: int, k: int, out: torch.Tensor,
                workspace: torch.Tensor | None = None) -> torch.Tensor:
     """Ordered top-k of every row of fp32 ``scores`` (n_rows, H, L); row n of head h
     lands at (n // rep)*seq_stride + h*head_stride + (n % rep)*rep_stride in ``out``.
-    ``lru`` = (page_access_time (H, N), candidates (H, k_cand) int32): the same launch
-    also lists the k_cand least recently used slots of every head, for the LRU
-    update that follows.  ``workspace``: candidate buffer for rows longer than
+    ``lru`` = (page_access_time (H, N), candidates (H, k_cand) int32 from
+    lru_kernel.candidate_list, current_step): the same launch also lists the k_cand
+    least recently used slots of every head, stamped with the step counter's value,
+    for the LRU update that follows.  ``workspace``: candidate buffer for rows longer than
     16384 pages (da_topk_pages_workspace_bytes); by default one per shape and stream
     is kept by this module."""
     n_rows, H, L = scores.shape
@@ -67,11 +68,15 @@ def topk_pages(scores: torch.Tensor, rep: int, k: int, out: torch.Tensor,
     if workspace is None and n_rows > 0 and k > 0 and L > 16384:
         workspace = _split_workspace(n_rows, H, L, k, scores.device)
     if lru is None:
-        time_ptr, time_hs, time_code, n_slots, k_cand, cand_ptr = None, 0, 0, 0, 0, None
+        time_ptr, time_hs, time_code, n_slots, k_cand, cand_ptr, step_ptr = None, 0, 0, 0, 0, None, None
     else:
-        access_time, candidates = lru
+        from .lru_kernel import check_candidate_list
+
+        access_time, candidates, current_step = lru
         assert access_time.shape[0] == H and candidates.shape[0] == H
-        assert candidates.dtype == torch.int32 and candidates.is_contiguous()
+        assert current_step.dtype == torch.int32
+        check_candidate_list(candidates)
+        step_ptr = current_step.data_ptr()
         time_ptr, time_hs = access_time.data_ptr(), access_time.stride(0)
         time_code, n_slots = _lib.time_code(access_time.dtype), access_time.shape[1]
         k_cand, cand_ptr = candidates.shape[1], candidates.data_ptr()
@@ -79,7 +84,7 @@ def topk_pages(scores: torch.Tensor, rep: int, k: int, out: torch.Tensor,
         lib.da_topk_pages_lru(
             scores.data_ptr(), scores.stride(0), scores.stride(1), n_rows, rep, H, L, k,
             out.data_ptr(), seq_stride, head_stride, rep_stride, _lib.itype_code(out.dtype),
-            time_ptr, time_hs, time_code, n_slots, k_cand, cand_ptr,
+            time_ptr, time_hs, time_code, n_slots, k_cand, cand_ptr, step_ptr,
             None if workspace is None else workspace.data_ptr(),
             0 if workspace is None else workspace.numel() * workspace.element_size(),
             _lib.stream_ptr(scores.device),

@@ -160,14 +160,19 @@ int da_topk_pages(const float *scores, int64_t row_stride, int64_t head_stride,
  * for.  Needs n_heads == Hkv; k_cand <= min(N_hbm, 8192); candidates == NULL or
  * k_cand == 0 gives plain da_topk_pages.  n_rows == 0 or kp == 0 with a list
  * requested computes the list only.
+ *   candidates : n_heads * k_cand + n_heads int32: the lists, (n_heads, k_cand),
+ *                followed by one stamp word per head
+ *   step       : the LRU step counter da_lru_update will be given (required with
+ *                a list); its value at the time of this launch is stored as the
+ *                stamp of every head's list
  */
 int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_t head_stride,
                       int n_rows, int rep, int n_heads, int64_t n_pages, int kp,
                       void *out, int64_t out_seq_stride, int64_t out_head_stride,
                       int64_t out_rep_stride, int out_itype, const void *access_time,
                       int64_t time_head_stride, int time_type, int n_hbm_pages, int k_cand,
-                      int32_t *candidates, void *workspace, size_t workspace_bytes,
-                      void *stream);
+                      int32_t *candidates, const int32_t *step, void *workspace,
+                      size_t workspace_bytes, void *stream);
 
 /*
  * Subsystem 4a — LRU lookup / touch / evict / slot-assign for one decode step.
@@ -183,14 +188,18 @@ int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_t head_stri
  *   hit_mask     : optional (Hkv, K) bytes, 1 = page was resident when visited
  *   miss_page/miss_slot : (Hkv, K) int32, the i-th distinct missed page of a
  *                  head and the slot it was given; miss_count : (Hkv) int32
- *   candidates   : optional (Hkv, k_cand) int32 from da_topk_pages_lru: the k_cand
- *                  least recently used slots of every head in eviction order, taken
- *                  after the previous da_lru_update and before this one.  The
- *                  kernel then finds its victims by dropping the slots this call
- *                  touches from that list instead of ordering all slots again (it
- *                  orders them itself whenever the list is too short); a list
- *                  that does not describe the current access times gives wrong
- *                  evictions (entries that are no slot number are ignored).
+ *   candidates   : optional, as da_topk_pages_lru writes it (Hkv lists of k_cand
+ *                  int32, then Hkv stamp words): the k_cand least recently used
+ *                  slots of every head in eviction order.  The kernel then finds
+ *                  its victims by dropping the slots this call touches from that
+ *                  list instead of ordering all slots again (it orders them itself
+ *                  whenever the list is too short).  A list is only used when its
+ *                  stamp equals *step as this call reads it and DA_LRU_BUMP_STEP is
+ *                  set: every bumping update changes the access times and the
+ *                  counter together, so a list made before an earlier update (a
+ *                  stale list) is recognised and ignored, with the same result as
+ *                  passing none; so is any list handed to a call that does not
+ *                  bump.  Entries that are no slot number are ignored.
  *                  NULL / k_cand = 0: no list.
  *   slot_epoch   : optional (Hkv, N_hbm) int32; a slot handed to a missed page
  *                  gets the step value, so a later kernel can tell which slots
@@ -370,6 +379,14 @@ typedef struct da_paged_overlap {
   void *hbm;
   int64_t hbm_head_stride_bytes, hbm_slot_stride_bytes;
   const int32_t *miss_page;       /* (Hkv, miss_capacity) */
+  /* DA_PHASE_STREAM only: two rates of the machine, in GB/s, from which the launch
+   * decides whether the page stream of a step is long enough to leave the first
+   * pass to a few workgroups per kv head (which then keep off the compute units
+   * the stream runs on).  link_gbps: what reads of the pinned store issued by a
+   * kernel reach over the host link; block_gbps: what one workgroup alone on its
+   * compute unit reads from HBM.  0 = the values of the box the library was tuned
+   * on (54 and 30).  They move time only: the results do not depend on them. */
+  float link_gbps, block_gbps;
 } da_paged_overlap;
 
 int da_decode_attention_paged(const void *q, int64_t q_head_stride, int n_q_heads,

@@ -350,13 +350,13 @@ def test_topk_pages_keys_that_differ_in_few_bits(family, k):
 def test_lru_candidates_at_late_steps(lo, hi, ttype):
     """Access times of a long decoding run (large step counts, a narrow window of them):
     the short list of least recent slots is still the head of the stable order."""
-    from dram_attention_amd.lru_kernel import LruScratch, lru_candidates
+    from dram_attention_amd.lru_kernel import LruScratch, candidate_list, lru_candidates
 
     H, N, kc = 2, 2048, 256
     time = torch.randint(lo, hi, (H, N), generator=gen(lo + hi)).to(ttype)
-    sc = LruScratch.allocate(H, 16, DEV, N)._replace(
-        candidates=torch.empty(H, kc, dtype=torch.int32, device=DEV))
-    got = lru_candidates(time.to(DEV), sc).cpu().long()
+    sc = LruScratch.allocate(H, 16, DEV, N)._replace(candidates=candidate_list(H, kc, DEV))
+    step = torch.tensor([hi], dtype=torch.int32, device=DEV)
+    got = lru_candidates(time.to(DEV), sc, step).cpu().long()
     assert same(got, torch.sort(time, dim=-1, stable=True).indices[:, :kc])
 
 
@@ -365,16 +365,20 @@ def test_lru_candidates_at_late_steps(lo, hi, ttype):
 def test_lru_candidates_are_the_stable_order_of_the_access_times(N, kc, ttype):
     """The candidate list is the head of argsort(access_time, stable=True), up to the
     complete order of all slots."""
-    from dram_attention_amd.lru_kernel import LruScratch, lru_candidates
+    from dram_attention_amd.lru_kernel import LruScratch, candidate_list, lru_candidates
 
     H = 3
     time = torch.randint(0, 900, (H, N), generator=gen(N + kc)).to(ttype)
     time[1] = 7                                  # one head with every slot tied
-    sc = LruScratch.allocate(H, 16, DEV, N)._replace(
-        candidates=torch.empty(H, kc, dtype=torch.int32, device=DEV))
-    got = lru_candidates(time.to(DEV), sc).cpu().long()
+    sc = LruScratch.allocate(H, 16, DEV, N)._replace(candidates=candidate_list(H, kc, DEV))
+    step = torch.tensor([901], dtype=torch.int32, device=DEV)
+    cand = lru_candidates(time.to(DEV), sc, step)
+    got = cand.cpu().long()
     want = torch.sort(time, dim=-1, stable=True).indices[:, :kc]
     assert same(got, want)
+    # every head's list carries the step counter's value as its stamp, behind the lists
+    stamps = torch.as_strided(cand, (H,), (1,), cand.storage_offset() + H * kc)
+    assert stamps.cpu().tolist() == [901] * H
 
 
 def test_empty_inputs_are_no_ops():
@@ -517,7 +521,7 @@ def test_load_lru_cache_when_the_step_ties_with_stored_times(itype, ttype):
 
 
 def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat16, page_dim=256,
-              hot=None, serial_walk=False, candidates=False):
+              hot=None, serial_walk=False, candidates=False, refresh_every=1):
     """Random request trace on LRUCache-like state; compares every buffer with the
     oracle's serial walk after every step."""
     from dram_attention_amd.lru_kernel import LruScratch, lru_candidates, lru_update_and_gather
@@ -541,8 +545,10 @@ def lru_trace(H, P, N, K, steps, seed, itype, ttype, pinned, dtype=torch.bfloat1
         else:
             idx = rng.integers(0, P, (H, K))
         hit_o, miss_o = O.lru_load(st, idx, s, as_np(dram), as_np(hbm_o))
-        if candidates:   # the least recent slots listed ahead of the update, as the module does
-            order = lru_candidates(time, scratch).cpu()
+        if candidates and (s - 1) % refresh_every:
+            pass             # the update below is handed the list of an earlier step
+        elif candidates:     # the least recent slots listed ahead of the update, as the module does
+            order = lru_candidates(time, scratch, step).cpu()
             want = torch.sort(time.cpu().float(), dim=1, stable=True).indices[:, :order.shape[1]]
             assert same(order.long(), want), f"candidates, step {s}"
         lru_update_and_gather(dram_dev, time, d2h, h2d, torch.from_numpy(idx).to(itype).to(DEV),
@@ -598,6 +604,20 @@ def test_lru_update_with_candidate_list_matches_serial_walk(H, P, N, K, ttype):
     lru_trace(H, P, N, K, 10, 400 + K, torch.int64, ttype, False, candidates=True)
     lru_trace(H, P, N, K, 10, 500 + K, torch.int64, ttype, False, hot=max(2, P // 8),
               candidates=True)
+
+
+@pytest.mark.parametrize("H,P,N,K,ttype", [
+    (8, 8192, 2048, 1024, torch.float32),     # the 128K layer
+    (2, 16384, 4096, 4096, torch.float32),    # the 1M layer's shape: the complete order as the list
+    (3, 300, 100, 37, torch.int32),
+])
+def test_lru_update_ignores_a_stale_candidate_list(H, P, N, K, ttype):
+    """A list of least recent slots made one or two updates ago no longer describes the
+    access times.  Its stamp (the step counter when it was made) says so: the update
+    orders the slots itself and ends in the serial walk's state, as without a list."""
+    lru_trace(H, P, N, K, 9, 600 + K, torch.int64, ttype, False, candidates=True, refresh_every=3)
+    lru_trace(H, P, N, K, 9, 700 + K, torch.int64, ttype, False, hot=max(2, P // 8),
+              candidates=True, refresh_every=3)
 
 
 def test_lru_update_forced_serial_walk_gives_the_same_state():

@@ -428,6 +428,42 @@ def test_stream_variants_agree_on_random_small_shapes(seed):
             assert same(m.cache_k, mods[0].cache_k)
 
 
+def test_machine_rates_of_the_stream_launch_move_time_only():
+    """The stream + attention launch reads two rates of the machine (host link, one
+    workgroup's HBM read rate) to decide how many workgroups compute the first pass
+    next to the page stream.  Both extremes (every step leaves the pass to a few
+    workgroups per kv head; no step does) give the same output, slots and cache rows
+    bit for bit; another count of stream workgroups cuts the miss list differently, so
+    the output agrees up to the order of the softmax merge and the state bit for bit."""
+    from dram_attention_amd import DRAMAttention
+
+    w = WORKLOADS["128k"].scaled(dram_tokens=32768, local_cache=2048, lru_tokens=8192,
+                                 top_k_tokens=1024, steps=5)
+    prompt = make_prompt(w, 9)
+    mods = []
+    for link, block, blocks in ((0.0, 0.0, 32), (1e-3, 1e6, 32), (1e6, 1e-3, 32), (54.0, 30.0, 16),
+                                (1e-3, 1e6, 64)):
+        m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                          w.n_kv_heads, w.head_dim, device=DEV, dtype=w.dtype)
+        m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
+        assert 10.0 < m.link_gbps < 200.0          # init_cache measured the box's link
+        m.link_gbps, m.block_gbps, m.stream_blocks = link, block, blocks
+        mods.append(m)
+    inputs = DecodeInputs(w, prompt.q0, 9)
+    for t in range(w.steps):
+        xq, xk, xv = (x.to(DEV) for x in inputs.next())
+        outs = [m(xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate") for m in mods]
+        torch.cuda.synchronize()
+        assert mods[0].lru_cache.last_miss_counts().sum().item() > 0
+        for m, out in zip(mods[1:], outs[1:]):
+            if m.stream_blocks == mods[0].stream_blocks:
+                assert same(out, outs[0]), f"step {t}"
+            else:
+                assert close(out.float(), outs[0].float(), 1e-2, 1e-2), f"step {t}"
+            assert same(m.lru_cache.hbm_kv_cache, mods[0].lru_cache.hbm_kv_cache)
+            assert same(m.cache_k, mods[0].cache_k) and same(m.cache_v, mods[0].cache_v)
+
+
 def test_page_stream_overlap_changes_nothing():
     """Attention issued around a concurrent page stream (two phases, side stream)
     gives the bits of the serialised order, and both agree with one plain pass."""
@@ -717,11 +753,13 @@ def test_static_prefix_equals_full_attention(full_size):
 
 
 # ------------------------------------------------------------ full size, by properties
-@pytest.mark.parametrize("name,steps", [("128k", 6), ("1m", 3)])
+@pytest.mark.parametrize("name,steps", [("128k", 6), ("1m", 64)])
 def test_full_size_invariants(name, steps):
     """configs[2] (128K prefix, 8192 pages/head) and configs[4] (1M prefix, 65536
-    pages/head, 64 query heads) at full size: invariants that need no CPU walk,
-    plus attention against a dense fp32 computation on the GPU."""
+    pages/head, 64 query heads; all of its 64 steps, in which every slot is handed
+    out several times over since a step requests as many pages as there are slots)
+    at full size: invariants that need no CPU walk, plus attention against a dense
+    fp32 computation on the GPU."""
     from dram_attention_amd import DRAMAttention
 
     w = WORKLOADS[name]
