@@ -43,33 +43,45 @@ def _hipcc() -> str:
     return exe
 
 
-def check_hand_placed_registers(verbose: bool = False) -> None:
-    """The tile scorer (csrc/page_score_tile.hpp) places a few vector instructions by
-    inline asm, which the compiler's tracking of matrix-core hazards does not see.
-    Its safety rule is that those instructions write only registers no MFMA of the
-    kernel ever names as an operand or destination.  This reads the compiler's own
-    listing of page_score.hip and fails the build if any variant breaks the rule."""
+def check_tile_scorer_listing(text: str) -> int:
+    """The rule the hand-placed instructions of the tile scorer (csrc/page_score_tile.hpp)
+    must keep, checked on the compiler's own listing ``text`` of page_score.hip; returns
+    the number of kernel variants checked and raises RuntimeError naming the kernel and
+    the offending line otherwise.
+
+    The scorer places its dot products by inline asm in blocks of eight, which the
+    compiler's tracking of matrix-core hazards does not see.  Per variant:
+      - the kernel starts by claiming eight registers (eight ``v_mov_b32 vN, 0``: the
+        first eight of the kernel) and has at least one MFMA;
+      - every ``v_dot2_f32_bf16`` sits in a run of exactly eight, each writing a
+        different one of the claimed registers, and the run is closed by ``s_nop 2``
+        (the wait a dot product's consumer needs);
+      - no claimed register is an operand or destination of an MFMA, unless every such
+        MFMA comes after the last hand-placed write to it, in straight-line code
+        (never inside a loop that also holds such a write)."""
     import re
 
-    hipcc = _hipcc()
-    listing = HERE / "build" / "page_score.s"
-    cmd = [hipcc, *[f for f in HIPCC_FLAGS if f != "-fPIC"], "-S", "--cuda-device-only",
-           str(CSRC / "page_score.hip"), "-o", str(listing)]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError(f"hipcc -S failed on page_score.hip:\n{proc.stderr}")
-    text = listing.read_text()
-    names = re.findall(r"^(_ZN2da22page_score_tile_kernel[^\s:]*):", text, re.M)
-    if not names:
+    heads = list(re.finditer(r"^(_ZN2da22page_score_tile_kernel[^\s:]*):", text, re.M))
+    if not heads:
         raise RuntimeError("no page_score_tile_kernel in the listing of page_score.hip")
-    for name in names:
-        start = text.index("\n" + name + ":")
+    names = [m.group(1) for m in heads]
+    for head in heads:
+        name, start = head.group(1), head.start()
         lines = text[start:text.index("s_endpgm", start)].splitlines()
-        placed, matrix, labels, loops = {}, {}, {}, []
+
+        def bad(n, why):
+            return RuntimeError(f"{name}: {why} (line {n} of the kernel: {lines[n].strip()!r})")
+
+        claimed, claim_line = [], {}
+        writes, matrix, labels, loops, dots = {}, {}, {}, [], []
         for n, line in enumerate(lines):
-            m = re.match(r"\s+(v_dot2_f32_bf16|v_bfi_b32|v_mov_b32) v(\d+),", line)
+            m = re.match(r"\s+v_mov_b32 v(\d+), 0\s*$", line)
+            if m and len(claimed) < 8 and not dots:
+                claimed.append(int(m.group(1)))
+                claim_line[int(m.group(1))] = n
+            m = re.match(r"\s+v_dot2_f32_bf16 v(\d+),", line)
             if m:
-                placed.setdefault(int(m.group(2)), []).append(n)
+                dots.append((n, int(m.group(1))))
             m = re.match(r"\s+v_mfma\S+ (.*)", line)
             if m:
                 for lo, hi in re.findall(r"v\[(\d+):(\d+)\]", m.group(1)):
@@ -83,21 +95,57 @@ def check_hand_placed_registers(verbose: bool = False) -> None:
                 target = labels.get(m.group(1) or m.group(2))
                 if target is not None:          # a label already seen: a backward branch, i.e. a loop
                     loops.append((target, n))
-        if len(placed) != 8 or not matrix:
-            raise RuntimeError(f"{name}: expected 8 hand-placed destinations and some MFMAs, "
-                               f"found {len(placed)} and {len(matrix)} registers")
+        if len(set(claimed)) != 8:
+            raise RuntimeError(f"{name}: expected eight registers claimed by v_mov_b32 vN, 0 ahead of "
+                               f"the first dot product, found {sorted(set(claimed))}")
+        if not matrix:
+            raise RuntimeError(f"{name}: no MFMA in the kernel")
+        if not dots or len(dots) % 8:
+            raise RuntimeError(f"{name}: {len(dots)} hand-placed dot products, not blocks of eight")
+        for b in range(0, len(dots), 8):
+            block = dots[b:b + 8]
+            first = block[0][0]
+            for i, (n, reg) in enumerate(block):
+                if n != first + i:
+                    raise bad(n, "a hand-placed dot product outside a run of eight")
+                if reg not in claimed:
+                    raise bad(n, f"a hand-placed dot product writes v{reg}, which the kernel never claimed")
+            if len({reg for _, reg in block}) != 8:
+                raise bad(first, "a block of dot products writes a register twice")
+            closing = first + 8
+            if closing >= len(lines) or not re.match(r"\s+s_nop 2\s*$", lines[closing]):
+                raise bad(min(closing, len(lines) - 1), "a block of dot products is not closed by s_nop 2")
+            for n, reg in block:
+                writes.setdefault(reg, []).append(n)
+        for reg in claimed:
+            writes.setdefault(reg, []).append(claim_line[reg])
         # A register may serve both only when every MFMA that names it comes after
         # the last hand-placed write to it (the variable behind it is dead by then),
         # in straight-line code: never inside a loop that also holds such a write.
-        for r in sorted(set(placed) & set(matrix)):
-            last_write, first_use = max(placed[r]), min(matrix[r])
+        for r in sorted(set(writes) & set(matrix)):
+            last_write, first_use = max(writes[r]), min(matrix[r])
             in_one_loop = any(lo <= w <= hi and lo <= u <= hi for lo, hi in loops
-                              for w in placed[r] for u in matrix[r])
+                              for w in writes[r] for u in matrix[r])
             if first_use < last_write or in_one_loop:
-                raise RuntimeError(f"{name}: register v{r} is written by a hand-placed "
-                                   "instruction while an MFMA may still use it")
+                raise bad(first_use, f"register v{r} is written by a hand-placed instruction while "
+                                     "an MFMA may still use it")
+    return len(names)
+
+
+def check_hand_placed_registers(verbose: bool = False) -> None:
+    """Compile page_score.hip to a listing and hold it against check_tile_scorer_listing;
+    fails the build if any variant of the tile scorer breaks the rule."""
+    hipcc = _hipcc()
+    (HERE / "build").mkdir(exist_ok=True)
+    listing = HERE / "build" / "page_score.s"
+    cmd = [hipcc, *[f for f in HIPCC_FLAGS if f != "-fPIC"], "-S", "--cuda-device-only",
+           str(CSRC / "page_score.hip"), "-o", str(listing)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc -S failed on page_score.hip:\n{proc.stderr}")
+    n = check_tile_scorer_listing(listing.read_text())
     if verbose:
-        print(f"hand-placed registers of {len(names)} tile scorer variants are clear of MFMA operands")
+        print(f"hand-placed registers of {n} tile scorer variants are clear of MFMA operands")
 
 
 def build_library(verbose: bool = False) -> Path:

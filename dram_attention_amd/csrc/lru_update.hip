@@ -424,14 +424,17 @@ extern "C" int da_lru_update(const void *idx, int64_t idx_head_stride, int idx_i
   // the stamp is the bumped step counter, which is; a caller-supplied stamp may tie
   // with stored times, and then only the literal walk gives the reference's result
   // (a slot hit earlier in the walk can be chosen as a victim later in it).
-  const bool stamp_may_tie = !bump_step && n_hbm_pages <= kSelMaxK;
+  const bool stamp_may_tie = !bump_step;
   const int serial = ((flags & DA_LRU_SERIAL_WALK) || k > n_hbm_pages || k > kLruMaxK ||
                       stamp_may_tie) ? 1 : 0;
   if (serial && n_hbm_pages > kSelMaxK)
     return fail(DA_ENOTSUP,
-                "da_lru_update: k %d > slots %d needs the serial walk, which orders at most %d "
-                "slots",
-                k, n_hbm_pages, kSelMaxK);
+                "da_lru_update: %s needs the serial walk, which orders at most %d slots (%d here)",
+                stamp_may_tie && k <= n_hbm_pages && !(flags & DA_LRU_SERIAL_WALK)
+                    ? "a caller-supplied time stamp (no DA_LRU_BUMP_STEP), which may tie with "
+                      "stored access times,"
+                    : "this call (more requests than slots, or DA_LRU_SERIAL_WALK)",
+                kSelMaxK, n_hbm_pages);
   dim3 grid(n_kv_heads);
   hipStream_t s = (hipStream_t)stream;
   int32_t *ticket = (int32_t *)workspace;

@@ -115,7 +115,7 @@ class IPUpperboundTopKSelector:
         # contents into chunk_min_max
         self.bounds_are_ordered = True
         self._scores = None
-        self._split_ws = {}     # candidate buffers of long rows, by (rows, k): this selector's own
+        self._split_ws = None   # candidate buffer of long rows: this selector's own, the largest so far
 
     def scores(self, q: torch.Tensor) -> torch.Tensor:
         """fp32 scores (seq_len*rep, num_kv_heads, num_pages); row s*rep + r is query
@@ -139,12 +139,18 @@ class IPUpperboundTopKSelector:
                            ordered_bounds=self.bounds_are_ordered)
 
     def _workspace(self, scores: torch.Tensor, k: int):
+        """Candidate buffer of the two-launch selection of rows beyond 16384 pages (None
+        when the shape needs none).  One buffer per selector, grown to the largest
+        shape seen and shared by the smaller ones; it carries nothing from call to call,
+        so the calls of one selector must follow each other on ONE stream (two streams
+        stepping the same selector would race on it)."""
         n_rows, H, L = scores.shape
-        if (n_rows, k) not in self._split_ws:
-            need = _lib.load().da_topk_pages_workspace_bytes(n_rows, H, L, k)
-            self._split_ws[(n_rows, k)] = (torch.empty(need, dtype=torch.uint8, device=scores.device)
-                                           if need else None)
-        return self._split_ws[(n_rows, k)]
+        need = _lib.load().da_topk_pages_workspace_bytes(n_rows, H, L, k)
+        if need == 0:
+            return None
+        if self._split_ws is None or self._split_ws.numel() < need:
+            self._split_ws = torch.empty(need, dtype=torch.uint8, device=scores.device)
+        return self._split_ws
 
     def top_k(self, q: torch.Tensor, k: int) -> torch.Tensor:
         """Indices of the top k pages, (seq_len, num_kv_heads, rep, k) int64, best first."""

@@ -208,8 +208,8 @@ int da_topk_pages_lru(const float *scores, int64_t row_stride, int64_t head_stri
  * N_hbm with DA_LRU_BUMP_STEP runs fully parallel, K > N_hbm falls back to one
  * serial lane per head.  Without DA_LRU_BUMP_STEP the time stamp is the
  * caller's *step and may tie with stored access times, where only the literal
- * walk is right: such calls take it too (with more than 8192 slots they stay
- * parallel and *step must then exceed every stored access time).
+ * walk is right: such calls take it too.  The walk orders at most 8192 slots
+ * per head: a call that needs it with more slots is refused (DA_ENOTSUP).
  * DA_LRU_SERIAL_WALK in `flags` takes that literal walk for any K (a checking
  * and benchmarking aid: the result is the same, only slower).
  * A miss_slot of -1 marks an entry whose slot was re-assigned later in the

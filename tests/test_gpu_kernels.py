@@ -741,3 +741,25 @@ def test_decode_attention_rejects_overflow_and_bad_dim():
         decode_attention(torch.zeros(4, 24, device=DEV), None, None,
                          torch.zeros(8, 2, 24, device=DEV), torch.zeros(8, 2, 24, device=DEV), 1,
                          None, None)
+
+
+def test_lru_update_with_a_caller_stamp_and_more_slots_than_the_walk_orders_is_refused():
+    """Without the step bump the stamp may tie with stored times and only the literal walk
+    is right; the walk orders at most 8192 slots per head, so such a call with more slots
+    is refused before any launch instead of running a form that could evict a slot it hit."""
+    from dram_attention_amd.lru_kernel import LruScratch, lru_update
+
+    H, P, N, K = 1, 20000, 9000, 8
+    dram = torch.zeros(H, P, 16, device=DEV)
+    hbm = torch.zeros(H, N, 16, device=DEV)
+    time = torch.zeros(H, N, device=DEV)
+    d2h = torch.full((H, P), -1, dtype=torch.int64, device=DEV)
+    h2d = torch.full((H, N), -1, dtype=torch.int64, device=DEV)
+    idx = torch.arange(K, device=DEV)[None]
+    step = torch.ones(1, dtype=torch.int32, device=DEV)
+    sc = LruScratch.allocate(H, K, DEV, N)
+    with pytest.raises(RuntimeError, match="caller-supplied time stamp"):
+        lru_update(dram, time, d2h, h2d, idx, step, hbm, sc, bump_step=False)
+    lru_update(dram, time, d2h, h2d, idx, step, hbm, sc, bump_step=True)      # the bumped form runs
+    torch.cuda.synchronize()
+    assert step.item() == 2 and sc.miss_count.item() == K

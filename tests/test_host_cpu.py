@@ -187,3 +187,60 @@ def test_bench_steps_per_graph_choice():
     for n in range(1, 200):
         spg = f(n, 32, 32)
         assert 1 <= spg <= min(n, 32) and (n % spg == 0 or spg == min(n, 32))
+
+
+def tile_scorer_listing(dot_regs=(1, 145, 142, 146, 143, 147, 144, 148), closing="s_nop 2",
+                        mfma="v_mfma_f32_16x16x32_bf16 v[166:169], v[170:173], v[90:93], v[166:169]",
+                        loop=False, stray_dot=False):
+    """A listing in the shape hipcc -S gives the tile scorer: eight claimed registers, one
+    block of eight hand-placed dot products, one MFMA; the arguments doctor it."""
+    claimed = (1, 145, 142, 146, 143, 147, 144, 148)
+    lines = ["_ZN2da22page_score_tile_kernelILi2ELi4ELi8ELb0EEEvPKcllS2_ilPfllii: ; @kernel",
+             "\ts_load_dwordx4 s[0:3], s[4:5], 0x0"]
+    lines += [f"\tv_mov_b32 v{r}, 0" for r in claimed]
+    lines += [".LBB9_1:", "\tv_perm_b32 v140, v10, v11, s6"]
+    lines += [f"\tv_dot2_f32_bf16 v{r}, v{178 + i}, v{157 + i}, 0" for i, r in enumerate(dot_regs)]
+    lines += [f"\t{closing}", "\tv_cvt_pk_bf16_f32 v170, v1, v145"]
+    if stray_dot:
+        lines += ["\tv_dot2_f32_bf16 v1, v140, v157, 0"]
+    lines += [f"\t{mfma}"]
+    if loop:
+        lines += ["\ts_cbranch_scc1 .LBB9_1"]
+    lines += ["\tglobal_store_dword v[2:3], v166, off", "\ts_endpgm"]
+    return "\n".join(lines) + "\n"
+
+
+def test_tile_scorer_hazard_check_on_doctored_listings():
+    """The build-time check of the tile scorer's hand-placed instructions accepts a
+    well-formed listing and refuses each way the rule can break: an MFMA that names a
+    hand-written register, a block that is not closed by its wait, a dot product that
+    writes an unclaimed register or sits outside a block of eight, a kernel with no
+    MFMA or no such kernel at all."""
+    from dram_attention_amd.build import check_tile_scorer_listing as check
+
+    assert check(tile_scorer_listing()) == 1
+    assert check(tile_scorer_listing() + tile_scorer_listing().replace("ILi2E", "ILi4E")) == 2
+    # an MFMA reads v142..v145 as its A operand ahead of a later hand-placed write (the loop)
+    with pytest.raises(RuntimeError, match="v142 is written by a hand-placed instruction"):
+        check(tile_scorer_listing(mfma="v_mfma_f32_16x16x32_bf16 v[166:169], v[142:145], v[90:93], v[166:169]",
+                                  loop=True))
+    # the same overlap as the MFMA's destination, straight-line but ahead of the last write
+    with pytest.raises(RuntimeError, match="v1 is written by a hand-placed instruction"):
+        check(tile_scorer_listing(mfma="v_mfma_f32_16x16x32_bf16 v[0:3], v[170:173], v[90:93], v[0:3]")
+              .replace("\tv_perm_b32 v140, v10, v11, s6",
+                       "\tv_mfma_f32_16x16x32_bf16 v[0:3], v[170:173], v[90:93], v[0:3]"))
+    with pytest.raises(RuntimeError, match="not closed by s_nop 2"):
+        check(tile_scorer_listing(closing="s_nop 1"))
+    with pytest.raises(RuntimeError, match="never claimed"):
+        check(tile_scorer_listing(dot_regs=(1, 145, 142, 146, 143, 147, 144, 149)))
+    with pytest.raises(RuntimeError, match="writes a register twice"):
+        check(tile_scorer_listing(dot_regs=(1, 145, 142, 146, 143, 147, 144, 144)))
+    with pytest.raises(RuntimeError, match="not blocks of eight"):
+        check(tile_scorer_listing(stray_dot=True))
+    with pytest.raises(RuntimeError, match="no MFMA"):
+        check(tile_scorer_listing(mfma="v_add_f32 v166, v170, v171"))
+    with pytest.raises(RuntimeError, match="no page_score_tile_kernel"):
+        check("_ZN2da21page_score_vec_kernelIfLi4EEEvv:\n\ts_endpgm\n")
+    # a claimed register may serve an MFMA once the hand-placed writes are over (no loop)
+    assert check(tile_scorer_listing(
+        mfma="v_mfma_f32_16x16x32_bf16 v[166:169], v[142:145], v[90:93], v[166:169]")) == 1
