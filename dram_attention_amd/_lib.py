@@ -27,6 +27,12 @@ SIGNATURES = {
     "da_version": (c_int, []),
     "da_last_error_string": (c_char_p, []),
     "da_host_device_pointer": (c_int, [c_void_p, ctypes.POINTER(c_void_p)]),
+    "da_prefill_attention": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64,
+         c_int64, c_int, c_int, c_int, c_int, c_float, c_void_p, c_int64, c_int64, c_void_p,
+         c_void_p],
+    ),
     "da_page_minmax": (
         c_int,
         [c_void_p, c_int64, c_int64, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p],

@@ -24,6 +24,7 @@ SOURCES = (
     "lru_update.hip",
     "decode_attention.hip",
     "stream_attention.hip",
+    "prefill_attention.hip",
 )
 # packed fp32 VALU ops are switched off for every device compile of this library
 HIPCC_FLAGS = (

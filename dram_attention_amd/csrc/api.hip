@@ -8,7 +8,7 @@ char *last_error_buffer() {
 }
 }  // namespace da
 
-extern "C" int da_version(void) { return 100; }
+extern "C" int da_version(void) { return 200; }
 
 extern "C" const char *da_last_error_string(void) { return da::last_error_buffer(); }
 

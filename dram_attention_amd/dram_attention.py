@@ -157,26 +157,72 @@ def decode_attention(
     return out
 
 
-def causal_prefill_attention(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor) -> torch.Tensor:
-    """Dense causal attention over the prompt, (1,S,Hq,D) -> (1,S,Hq,D).  Not on
-    the decode path; torch's fused SDPA stands in for flash_attn_func
-    (reference dram_attention.py:136).  If no fused kernel takes the shape,
-    queries go in blocks so that no S x S score matrix is ever materialised."""
-    from torch.nn.attention import SDPBackend, sdpa_kernel
+def prefill_attention_supported(xq: torch.Tensor) -> bool:
+    """Whether the library's own causal prefill kernel takes this query tensor."""
+    return (xq.is_cuda and xq.dtype in (torch.bfloat16, torch.float16)
+            and xq.shape[-1] in (64, 128))
 
+
+def prefill_attention(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor, *,
+                      scale: float | None = None, lse: torch.Tensor | None = None) -> torch.Tensor:
+    """Causal attention over the prompt on the library's kernel (da_prefill_attention):
+    (1,S,Hq,D), (1,S,Hkv,D) x 2 -> (1,S,Hq,D); fills ``lse`` (Hq, S) fp32 when given.
+    Replaces flash_attn_func(xq, xk, xv, causal=True), reference dram_attention.py:136."""
+    bsz, S, Hq, D = xq.shape
+    assert bsz == 1, "Only support batch size 1"
+    Hkv = xk.shape[2]
+    for name, t in (("xq", xq), ("xk", xk), ("xv", xv)):
+        _lib.require_gpu(t, name)
+        if t.stride(-1) != 1:
+            raise ValueError("head_dim must be the dense axis of every operand")
+    if xk.shape != xv.shape or xk.shape[1] != S or xk.shape[3] != D or not (
+            xq.dtype == xk.dtype == xv.dtype):
+        raise ValueError("query, keys and values must agree in length, head size and type")
+    out = torch.empty(1, S, Hq, D, dtype=xq.dtype, device=xq.device)
+    if lse is not None and (lse.shape != (Hq, S) or lse.dtype != torch.float32
+                            or not lse.is_contiguous()):
+        raise ValueError("lse must be a contiguous fp32 tensor of shape (Hq, S)")
+    _lib.check(
+        _lib.load().da_prefill_attention(
+            xq.data_ptr(), xq.stride(1), xq.stride(2), xk.data_ptr(), xk.stride(1), xk.stride(2),
+            xv.data_ptr(), xv.stride(1), xv.stride(2), S, Hq, Hkv, D, _lib.dtype_code(xq.dtype),
+            float(scale) if scale is not None else 1.0 / math.sqrt(D), out.data_ptr(),
+            out.stride(1), out.stride(2), lse.data_ptr() if lse is not None else None,
+            _lib.stream_ptr(xq.device)),
+        "da_prefill_attention")
+    return out
+
+
+def causal_prefill_attention(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor,
+                             backend: str = "auto") -> torch.Tensor:
+    """Dense causal attention over the prompt, (1,S,Hq,D) -> (1,S,Hq,D), in place of
+    flash_attn_func (reference dram_attention.py:136).  ``backend``:
+      "native"  the library's kernel (16-bit types, head_dim 64 or 128; raises otherwise)
+      "sdpa"    torch's fused scaled_dot_product_attention (raises if no fused kernel
+                takes the shape)
+      "blocked" torch's attention over blocks of 1024 query rows with an explicit mask,
+                so that no S x S score matrix is ever materialised (any type, CPU too)
+      "auto"    native where it applies, else sdpa, else blocked."""
+    if backend not in ("auto", "native", "sdpa", "blocked"):
+        raise RuntimeError(f"Unsupported prefill backend: {backend}")
+    if backend == "native" or (backend == "auto" and prefill_attention_supported(xq)):
+        return prefill_attention(xq, xk, xv)
     bsz, S, Hq, D = xq.shape
     Hkv = xk.shape[2]
     q = xq.transpose(1, 2)
     k = xk.transpose(1, 2)
     v = xv.transpose(1, 2)
     gqa = Hq != Hkv
-    if xq.is_cuda:
+    if backend == "sdpa" or (backend == "auto" and xq.is_cuda):
+        from torch.nn.attention import SDPBackend, sdpa_kernel
+
         try:
             with sdpa_kernel([SDPBackend.FLASH_ATTENTION, SDPBackend.EFFICIENT_ATTENTION]):
                 o = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=gqa)
             return o.transpose(1, 2).contiguous()
         except RuntimeError:
-            pass
+            if backend == "sdpa":
+                raise
     out = torch.empty_like(xq)
     block = 1024
     for s0 in range(0, S, block):
@@ -249,6 +295,8 @@ class DRAMAttention(torch.nn.Module):
         # of a copy engine's rate) and what one workgroup alone reads from HBM (0 = the
         # library's default).  Results do not depend on any of the three.
         self.stream_blocks = GATHER_BLOCKS
+        # which implementation stage="prefill" attends with: see causal_prefill_attention
+        self.prefill_backend = "auto"
         self.link_gbps = 0.0
         self.block_gbps = 0.0
 
@@ -326,7 +374,7 @@ class DRAMAttention(torch.nn.Module):
         bsz, seqlen, H, D = xq.shape
         assert bsz == 1, "Only support batch size 1"
         if stage == "prefill":
-            output = causal_prefill_attention(xq, xk, xv)
+            output = causal_prefill_attention(xq, xk, xv, self.prefill_backend)
             self.init_cache(xk, xv)
             return output
         elif stage == "generate":

@@ -58,6 +58,27 @@ const char *da_last_error_string(void);
 int da_host_device_pointer(const void *host_ptr, void **device_ptr);
 
 /*
+ * Prefill — causal attention over the whole prompt, one query row per prompt
+ * token: out[t, j, :] = softmax_{s <= t}(q[t, j, :] . k[s, j / rep, :] * scale) v[s, j / rep, :].
+ * Replaces flash_attn_func(xq, xk, xv, causal=True) in
+ * dram_attention/dram_attention.py:136 (batch 1, as the module asserts, :128).
+ *   q, out : (S, Hq, D), element strides (tok_stride, head_stride, 1)
+ *   k, v   : (S, Hkv, D) likewise; query head j reads kv head j / (Hq / Hkv)
+ *   scale  : softmax scale (flash-attn's default is D^-0.5), positive
+ *   lse_out: optional (Hq, S) fp32, natural log of the softmax denominator
+ * bf16 or fp16 with head_dim 64 or 128 (DA_ENOTSUP otherwise): tiled flash
+ * attention with both products on the matrix cores, fp32 accumulation, the
+ * softmax weights rounded to the input type for the second product (as
+ * flash-attn rounds them).  No workspace.
+ */
+int da_prefill_attention(const void *q, int64_t q_tok_stride, int64_t q_head_stride,
+                         const void *k, int64_t k_tok_stride, int64_t k_head_stride,
+                         const void *v, int64_t v_tok_stride, int64_t v_head_stride,
+                         int64_t seq_len, int n_q_heads, int n_kv_heads, int head_dim,
+                         int dtype, float scale, void *out, int64_t o_tok_stride,
+                         int64_t o_head_stride, float *lse_out, void *stream);
+
+/*
  * Subsystem 1 — per-page, per-channel min and max of the keys.
  * Replaces torch.aminmax + torch.stack in
  * dram_attention/topk_selector.py:31-34.
