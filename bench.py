@@ -33,6 +33,27 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0          # dense bf16 / fp16
+# HBM bytes per launch of the roofline kernel (first attention pass) from the committed
+# counter runs, by workload: the fallback when the summary file is not next to this script;
+# a CPU test holds it equal to what the file says.
+TRAFFIC_PROFILE = os.path.join("profiles", "bench_128k_hbm_traffic_pmc.md")
+ROOFLINE_TRAFFIC_BYTES = {"128k": 152.8e6}
+
+
+def roofline_traffic_from_profile(path=None):
+    """The 'HBM traffic of the roofline kernel per launch = ... = N MB' figure of the
+    committed counter summary, in bytes; None if the file is not there."""
+    import re
+
+    path = path or os.path.join(ROOT, TRAFFIC_PROFILE)
+    try:
+        with open(path) as f:
+            text = f.read()
+    except OSError:
+        return None
+    m = re.search(r"HBM traffic of the roofline kernel per launch\s*=[^\n]*?=\s*([0-9.]+)\s*MB", text)
+    return float(m.group(1)) * 1e6 if m else None
 WORKLOAD_INDEX = {"cpu": 0, "32k": 1, "128k": 2, "1m": 4}
 
 
@@ -69,6 +90,12 @@ def parse_args():
                     help="also time an attention-only stack of this many layers of the workload "
                          "(configs[3] at 32 with workload 128k), pipelined and serial; 0 = skip")
     ap.add_argument("--stack-steps", type=int, default=6, help="timed model steps of that stack")
+    ap.add_argument("--prefill-reps", type=int, default=2,
+                    help="also time causal prefill attention at the workload's prompt length, this "
+                         "library's kernel and torch's fused op; 0 = skip")
+    ap.add_argument("--no-value-64", action="store_true",
+                    help="skip the second timed run at the configuration's own 64 steps (warm-up 8) that "
+                         "is made when --steps/--warmup differ from it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 128 MiB device copy (reference point for HBM traffic counters)")
     return ap.parse_args()
@@ -77,7 +104,8 @@ def parse_args():
 class Layer:
     """One attention layer set up on the workload, plus the staged step inputs."""
 
-    def __init__(self, w, seed, total_steps, dev, overlap, force_lru=False, device_prompt=False):
+    def __init__(self, w, seed, total_steps, dev, overlap, force_lru=False, device_prompt=False,
+                 prompt=None):
         from dram_attention_amd import DRAMAttention, DummyCache, LRUCache
         from dram_attention_amd.synthetic import DecodeInputs, make_prompt
 
@@ -94,7 +122,8 @@ class Layer:
             self.m.init_cache(prompt.k, prompt.v)
             prompt.k = prompt.v = None
         else:
-            prompt = make_prompt(w, seed)
+            if prompt is None:
+                prompt = make_prompt(w, seed)
             self.m.init_cache(prompt.k.to(dev), prompt.v.to(dev))
         self.prompt = prompt
         if force_lru and isinstance(self.m.lru_cache, DummyCache):
@@ -347,6 +376,104 @@ def time_kernels(layer, steps):
     if "split+merge" in us:
         us["decode_attention_merge"] = us.pop("split+merge") - us["decode_attention_split"]
     return us, misses / steps, sum(local_rows) / len(local_rows)
+
+
+def time_step_launch(layer, steps):
+    """The launch that dominates a step, timed where it runs: `steps` further decode steps
+    issued as the module issues them (selection, then page stream + first attention pass
+    as ONE launch, then the merge), with an event on either side of the stream + attention
+    launch and a busy kernel ahead so that the launches are queued when the GPU gets to
+    them.  Returns (average us of that launch, average distinct misses per step)."""
+    m = layer.m
+    spent, misses = 0.0, 0
+    for _ in range(steps):
+        t = int(layer.t_dev.item())
+        xq, xk, xv = layer.qs[t:t + 1], layer.ks[t:t + 1], layer.vs[t:t + 1]
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda._sleep(2_000_000)
+        selected = m.select_(xq)
+        e0.record()
+        out, merge = m.attend_(xq, xk, xv, layer.pos_dev, selected, defer_merge=True)
+        e1.record()
+        if merge is None:
+            return None, None          # this shape does not take the one-launch form
+        merge()
+        torch.cuda.synchronize()
+        spent += e0.elapsed_time(e1)
+        misses += int(m.lru_cache.last_miss_counts().sum().item())
+        layer.cnt += 1
+    return spent / steps * 1e3, misses / steps
+
+
+def timed_replays(layer, steps, warmup, wanted_spg):
+    """`warmup` untimed + `steps` timed decode steps of a freshly built layer, captured and
+    replayed as the main leg does; returns (steps/s, steps per graph)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            layer.step_from_device_state()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    single = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(single):
+        layer.step_from_device_state()
+    spg = steps_per_graph(steps, wanted_spg, Layer.MAX_STEPS_PER_GRAPH)
+    many = None
+    if spg > 1:
+        many = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(many):
+            layer.steps_from_device_state(spg)
+    for _ in range(max(warmup - 2, 0)):
+        single.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps // spg if many is not None else 0):
+        many.replay()
+    for _ in range(steps % spg if many is not None else steps):
+        single.replay()
+    torch.cuda.synchronize()
+    return steps / (time.perf_counter() - t0), spg
+
+
+def prefill_leg(w, dev, reps, seed):
+    """stage="prefill" attention at the workload's prompt length: the library's kernel
+    (da_prefill_attention) and torch's fused op beside it, events on the launch stream;
+    flops = the causal half of two S x S x D products per query head."""
+    from dram_attention_amd.dram_attention import causal_prefill_attention, prefill_attention_supported
+
+    S, Hq, Hkv, D = w.prompt_tokens, w.n_q_heads, w.n_kv_heads, w.head_dim
+    g = torch.Generator(device=dev).manual_seed(seed)
+    xq = torch.randn(1, S, Hq, D, device=dev, generator=g).to(w.dtype)
+    xk = torch.randn(1, S, Hkv, D, device=dev, generator=g).to(w.dtype)
+    xv = torch.randn(1, S, Hkv, D, device=dev, generator=g).to(w.dtype)
+    flops = 4.0 * S * S * D * Hq / 2
+    res = {"prompt_tokens": S, "flops": flops, "reps": reps,
+           "what": "causal attention of stage=prefill (reference dram_attention.py:136), outside the "
+                   "decode-step metric; flops = 4*S*S*D*Hq/2"}
+    backends = (["native"] if prefill_attention_supported(xq) else []) + ["sdpa"]
+    for b in backends:
+        try:
+            causal_prefill_attention(xq, xk, xv, b)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                causal_prefill_attention(xq, xk, xv, b)
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / reps
+            tf = flops / (ms * 1e-3) / 1e12
+            res[b] = {"ms": ms, "TFLOPs": tf}
+            if b == "native":
+                res[b]["roofline"] = {"bound": "mfma", "kernel": "prefill_attention_kernel", "achieved": tf,
+                                      "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                      "frac": tf / MFMA_PEAK_TFLOPS}
+        except RuntimeError as exc:
+            res[b] = {"error": str(exc)[:200]}
+    if "native" in res and "sdpa" in res and "ms" in res["native"] and "ms" in res["sdpa"]:
+        res["native_over_sdpa"] = res["sdpa"]["ms"] / res["native"]["ms"]
+    return res
 
 
 def host_link_gbps(dev, mb=64, reps=5):
@@ -695,7 +822,8 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     w = WORKLOADS[args.workload]
-    total = args.warmup + args.steps + args.profile_steps + 4
+    step_launch_steps = 8
+    total = args.warmup + args.steps + args.profile_steps + step_launch_steps + 4
     layer = Layer(w, args.seed, total, dev, overlap=not args.no_overlap, force_lru=args.force_lru)
     if args.plain_scorer and isinstance(layer.m.lru_cache, LRUCache):
         layer.m.lru_cache.top_k_selector.bounds_are_ordered = False
@@ -746,7 +874,10 @@ def main():
     dt = time.perf_counter() - t0
     ms_per_step = dt / (args.steps * n_layers) * 1e3
 
-    # -- per-kernel pass and traffic counters
+    # -- the step's dominant launch where it runs, then every kernel alone, and traffic counters
+    paged = isinstance(layer.m.lru_cache, LRUCache)
+    step_launch_us, step_launch_misses = (time_step_launch(layer, step_launch_steps)
+                                          if paged and not args.no_overlap else (None, None))
     kernel_us, miss_per_step, local_rows = time_kernels(layer, args.profile_steps)
     score_b, attn_b = algorithmic_bytes(w, local_rows)
     attn_us = kernel_us["decode_attention_split"]
@@ -768,8 +899,9 @@ def main():
     # HBM bytes per launch of the roofline kernel from the committed counter runs
     # (profiles/bench_128k_hbm_traffic_pmc.md: FETCH_SIZE x 2.0 + WRITE_SIZE); only
     # known for the workload those runs used
-    traffic = 152.8e6 if w.name == "128k" else None
-    paged = isinstance(layer.m.lru_cache, LRUCache)
+    traffic = None
+    if w.name in ROOFLINE_TRAFFIC_BYTES:
+        traffic = roofline_traffic_from_profile() or ROOFLINE_TRAFFIC_BYTES[w.name]
     result = {
         "metric": "decode steps/sec per layer at 128K ctx; scorer+attn HBM GB/s vs peak",
         "value": args.steps * n_layers / dt,
@@ -810,6 +942,7 @@ def main():
                                if traffic is not None else None),
             "algorithmic_bytes": attn_b, "avg_us": attn_us,
         },
+        "roofline_step": None,
         "kernels_us": kernel_us,
         "kernels_us_note": "each kernel alone, after the timed region: 8 launches back to back between two "
                            "events, except lru_update, which changes its state and is one launch between "
@@ -822,6 +955,22 @@ def main():
                         "frac_of_link": stream_gbps / link if link else None,
                         "hit_rate": 1.0 - miss_per_step / requests},
     }
+    if step_launch_us:
+        step_bytes = step_launch_misses * page_bytes
+        step_gbps = step_bytes / (step_launch_us * 1e-6) / 1e9
+        result["roofline_step"] = {
+            "kernel": "decode_stream_attend_tile_kernel (page stream + first attention pass, the launch "
+                      "that dominates the timed step)" if w.dtype != torch.float32 else
+                      "decode_stream_attend_kernel (page stream + first attention pass)",
+            "bound": "host link", "bytes": step_bytes, "distinct_misses_per_step": step_launch_misses,
+            "avg_us": step_launch_us, "achieved": step_gbps, "peak": link, "unit": "GB/s",
+            "frac": step_gbps / link if link else None,
+            "peak_source": "pinned hipMemcpyAsync rate measured in this run",
+            "note": "events around the launch inside eagerly issued steps (selection before it, merge "
+                    "after it), 8 steps after the timed region",
+        }
+    else:
+        del result["roofline_step"]
     # The auxiliary legs below must never cost the headline line: a failure in one of
     # them is reported in its place.
     def leg(name, fn):
@@ -834,6 +983,26 @@ def main():
             print(f"bench.py: leg {name} failed: {type(exc).__name__}: {exc}", file=sys.stderr, flush=True)
 
     leg("cache_build", lambda: time_cache_build(layer, dev))
+    config_steps, config_warmup = w.steps, 8
+    if (args.steps, args.warmup) == (config_steps, config_warmup) or args.eager:
+        if not args.eager:
+            result["value_64"] = {"value": result["value"], "steps": config_steps, "warmup": config_warmup,
+                                  "note": "the timed region of this run"}
+    elif not args.no_value_64:
+        def value_64():
+            prompt = layer.prompt
+            l2 = Layer(w, args.seed, config_warmup + config_steps + 4, dev, overlap=not args.no_overlap,
+                       force_lru=args.force_lru, prompt=prompt)
+            if args.plain_scorer and isinstance(l2.m.lru_cache, LRUCache):
+                l2.m.lru_cache.top_k_selector.bounds_are_ordered = False
+            v, spg2 = timed_replays(l2, config_steps, config_warmup, args.steps_per_graph)
+            return {"value": v, "unit": "decode steps/s per layer", "steps": config_steps,
+                    "warmup": config_warmup, "ms_per_step": 1e3 / v, "steps_per_graph": spg2,
+                    "note": f"the configuration's own {config_steps} decode steps after {config_warmup} "
+                            "warm-up steps, same prompt and seed, a second layer built for it"}
+        leg("value_64", value_64)
+    if args.prefill_reps > 0 and w.dtype != torch.float32:
+        leg("prefill", lambda: prefill_leg(w, dev, args.prefill_reps, args.seed))
     if args.cpu_steps > 0:
         leg("cpu_baseline", lambda: cpu_baseline(w, args.seed, args.cpu_steps, prompt=layer.prompt))
     if args.reference_shaped_steps > 3 and isinstance(layer.m.lru_cache, LRUCache):

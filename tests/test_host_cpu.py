@@ -244,3 +244,17 @@ def test_tile_scorer_hazard_check_on_doctored_listings():
     # a claimed register may serve an MFMA once the hand-placed writes are over (no loop)
     assert check(tile_scorer_listing(
         mfma="v_mfma_f32_16x16x32_bf16 v[166:169], v[142:145], v[90:93], v[166:169]")) == 1
+
+
+def test_bench_roofline_traffic_constant_matches_the_committed_counter_summary():
+    """bench.py reports the roofline kernel's HBM bytes per launch from the committed
+    counter summary and keeps the same figure as a constant for when the file is not
+    beside it: the two must agree, so a refreshed profile cannot leave a stale constant."""
+    import bench
+
+    path = os.path.join(ROOT, bench.TRAFFIC_PROFILE)
+    assert os.path.exists(path)
+    parsed = bench.roofline_traffic_from_profile(path)
+    assert parsed is not None and parsed == bench.ROOFLINE_TRAFFIC_BYTES["128k"]
+    assert 151.26e6 <= parsed < 1.1 * 151.26e6      # at least the algorithmic bytes, little more
+    assert bench.roofline_traffic_from_profile(os.path.join(ROOT, "profiles", "no_such_file.md")) is None
