@@ -11,7 +11,7 @@ import torch
 from dram_attention_amd.synthetic import WORKLOADS, DecodeInputs, make_prompt
 from oracle import dram_attention_oracle as O
 
-from tests.parity import check_step
+from tests.parity import check_invariants, check_step
 from tests.util import close, same
 
 pytestmark = pytest.mark.gpu
@@ -763,51 +763,14 @@ def test_full_size_invariants(name, steps):
     from dram_attention_amd import DRAMAttention
 
     w = WORKLOADS[name]
-    H, rep, kp, D = w.n_kv_heads, w.rep, w.pages_per_q_head, w.head_dim
     prompt = make_prompt(w, 0)
     m = DRAMAttention(w.steps, w.lru_tokens, w.local_cache, 16, w.top_k_tokens, w.n_kv_heads,
                       w.head_dim, device=DEV, dtype=w.dtype)
     m.init_cache(prompt.k.to(DEV), prompt.v.to(DEV))
-    lru = m.lru_cache
-    dram_dev = lru.dram_kv_cache.to(DEV)
+    dram_dev = m.lru_cache.dram_kv_cache.to(DEV)
     inputs = DecodeInputs(w, prompt.q0, 0)
-    N, P = w.n_hbm_pages, w.n_dram_pages
-    ar = torch.arange(N, device=DEV)
     for t in range(steps):
         xq, xk, xv = inputs.next()
         xq, xk, xv = xq.to(DEV), xk.to(DEV), xv.to(DEV)
         out = m(xq, xk, xv, start_pos=w.prompt_tokens + t, stage="generate")
-        idx, d2h, h2d = lru._topk_idx, lru.dram_page_to_hbm_page_mapping, lru.hbm_page_to_dram_page_mapping
-        assert idx.shape == (H, rep * kp)
-        # selection: sorted by (score desc, index asc) within each query head, and no
-        # unselected page beats the last selected one
-        scores = lru.top_k_selector._scores                         # (rep, H, P)
-        sel = idx.view(H, rep, kp)
-        s_sel = torch.gather(scores.transpose(0, 1), 2, sel)          # (H, rep, kp)
-        assert torch.all((s_sel[..., :-1] > s_sel[..., 1:]) |
-                         ((s_sel[..., :-1] == s_sel[..., 1:]) & (sel[..., :-1] < sel[..., 1:])))
-        mask = torch.ones(H, rep, P, dtype=torch.bool, device=DEV).scatter_(2, sel, False)
-        rest = scores.transpose(0, 1).masked_fill(~mask, -float("inf"))
-        best_rest, best_idx = rest.max(dim=-1)
-        last, last_idx = s_sel[..., -1], sel[..., -1]
-        assert torch.all((best_rest < last) | ((best_rest == last) & (best_idx > last_idx)))
-        # LRU maps: inverse of each other, all requests resident and touched now
-        assert same(torch.gather(d2h, 1, h2d), ar.expand(H, N))
-        assert (d2h >= 0).sum().item() == H * N
-        slots = torch.gather(d2h, 1, idx)
-        assert torch.all(slots >= 0)
-        assert torch.all(torch.gather(lru.page_access_time, 1, slots) == t + 1)
-        assert lru.current_step.item() == t + 1
-        # payload: every slot holds exactly the page the map names
-        want_pages = torch.gather(dram_dev, 1, h2d[:, :, None].expand(-1, -1, dram_dev.shape[2]))
-        assert same(lru.hbm_kv_cache, want_pages)
-        # attention over all resident slots ++ local window ++ new token
-        c = w.prompt_tokens + t - w.dram_tokens
-        kk = torch.cat([lru.hbm_kv_cache.view(H, N * 16, 2, D)[:, :, 0],
-                        m.cache_k[0, : c + 1].transpose(0, 1)], 1).float()
-        vv = torch.cat([lru.hbm_kv_cache.view(H, N * 16, 2, D)[:, :, 1],
-                        m.cache_v[0, : c + 1].transpose(0, 1)], 1).float()
-        s = torch.einsum("hrd,htd->hrt", xq[0, 0].float().view(H, rep, D), kk) / math.sqrt(D)
-        want = torch.einsum("hrt,htd->hrd", torch.softmax(s, -1), vv).reshape(H * rep, D)
-        assert close(out[0, 0].float(), want, 2e-2, 1e-2)
-        assert same(m.cache_k[0, c], xk[0, 0]) and same(m.cache_v[0, c], xv[0, 0])
+        check_invariants(m, w, xq, xk, xv, out, t, dram_dev)

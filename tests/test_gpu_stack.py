@@ -12,7 +12,7 @@ import torch
 
 from dram_attention_amd.synthetic import WORKLOADS, DecodeInputs, make_prompt
 from oracle import dram_attention_oracle as O
-from tests.parity import check_step
+from tests.parity import check_invariants, check_step
 from tests.util import same
 
 pytestmark = pytest.mark.gpu
@@ -102,6 +102,85 @@ def test_pipelined_stack_matches_oracles_and_serial_order(shape):
         torch.cuda.synchronize()
         assert pos.item() == w.prompt_tokens + t + 1
         check(t, outs)
+
+
+def test_stack_of_32_full_size_layers_by_properties():
+    """configs[3] at its stated depth: 32 layers of the 128K shape (17 GB of pinned pages),
+    one model step per HIP graph, 9 decode steps.  No CPU walk: every layer of the
+    pipelined stack is held to the size-independent properties of a step (selection
+    ordered and maximal, maps mutually inverse, slot payload = mapped page, attention
+    against a dense fp32 softmax on the GPU), and to the bits of a second stack over the
+    same prompts whose layers are stepped one after the other on one stream."""
+    from dram_attention_amd import AttentionStack, DRAMAttention
+
+    w, n_layers, steps = WORKLOADS["128k"], 32, 9
+    Hq, Hkv, D = w.n_q_heads, w.n_kv_heads, w.head_dim
+    g = torch.Generator(device=DEV).manual_seed(77)
+    piped, serial, stores = [], [], []
+    for li in range(n_layers):
+        # the workload's distributions drawn on the GPU: K ~ N(0,1) x per-channel lognormal(0, 0.5)
+        k = torch.randn(w.prompt_tokens, Hkv, D, generator=g, device=DEV)
+        k *= torch.exp(0.5 * torch.randn(Hkv, D, generator=g, device=DEV))
+        k = k.to(w.dtype)[None]
+        v = torch.randn(w.prompt_tokens, Hkv, D, generator=g, device=DEV).to(w.dtype)[None]
+        for group in (piped, serial):
+            m = DRAMAttention(steps, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                              Hkv, D, device=DEV, dtype=w.dtype)
+            m.init_cache(k, v)
+            group.append(m)
+        stores.append(piped[-1].lru_cache.dram_kv_cache.to(DEV))
+        del k, v
+        if (li + 1) % 8 == 0:
+            print(f"stack test: {li + 1} of {n_layers} layer pairs built", flush=True)
+    stack, serial_stack = AttentionStack(piped, pipelined=True), AttentionStack(serial, pipelined=False)
+    # drifting queries as in the workload: q_t = 0.9 q_{t-1} + 0.44 N(0,1), per layer
+    q = torch.randn(n_layers, Hq, D, generator=g, device=DEV)
+    feeds = []
+    for t in range(steps):
+        if t:
+            q = 0.9 * q + 0.44 * torch.randn(n_layers, Hq, D, generator=g, device=DEV)
+        feeds.append((q.to(w.dtype), torch.randn(n_layers, Hkv, D, generator=g, device=DEV).to(w.dtype),
+                      torch.randn(n_layers, Hkv, D, generator=g, device=DEV).to(w.dtype)))
+    bufs = tuple(torch.empty_like(x) for x in feeds[0])
+    pos = torch.tensor([w.prompt_tokens], dtype=torch.int32, device=DEV)
+
+    def split(x):
+        return [x[li][None, None] for li in range(n_layers)]
+
+    def model_step():
+        return stack.generate(split(bufs[0]), split(bufs[1]), split(bufs[2]), pos)
+
+    def check(t, outs):
+        want = serial_stack.generate(*[split(x) for x in feeds[t]], w.prompt_tokens + t)
+        torch.cuda.synchronize()
+        missed = 0
+        for li in range(n_layers):
+            check_invariants(piped[li], w, *[x[li][None, None] for x in feeds[t]], outs[li], t,
+                             stores[li])
+            assert same(outs[li], want[li]), f"layer {li} step {t}: pipelined vs serial order"
+            assert same(piped[li].lru_cache.hbm_kv_cache, serial[li].lru_cache.hbm_kv_cache)
+            assert same(piped[li].lru_cache.page_access_time, serial[li].lru_cache.page_access_time)
+            missed += piped[li].lru_cache.last_miss_counts().sum().item()
+        assert missed > n_layers * 100          # the steps really paged
+
+    for dst, src in zip(bufs, feeds[0]):
+        dst.copy_(src)
+    outs = model_step()                         # step 0 eagerly: pinned mappings, workspaces
+    check(0, outs)
+    pos += 1
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = model_step()
+        pos += 1
+    for t in range(1, steps):
+        for dst, src in zip(bufs, feeds[t]):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert pos.item() == w.prompt_tokens + t + 1
+        check(t, outs)
+        print(f"stack test: step {t} of {steps - 1} checked", flush=True)
 
 
 def test_stack_argument_checks_and_short_stacks():
