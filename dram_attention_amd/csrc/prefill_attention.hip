@@ -147,16 +147,30 @@ prefill_attention_kernel(const PrefillArgs a) {
   const char *vbase = a.v + (int64_t)hk * a.v_head_stride * T::kBytes;
   const int64_t k_tok_b = a.k_tok_stride * T::kBytes, v_tok_b = a.v_tok_stride * T::kBytes;
 
+  // This thread's 16-byte chunks of a tile: chunk tid + 256*u = row tid/kRowChunks + u*(256/kRowChunks),
+  // column tid%kRowChunks.  Offsets inside a tile fit 32 bits (checked by the launcher).
   u32x4 kst[kLoads], vst[kLoads];
+  constexpr int kRowsPerLoad = kPfThreads / kRowChunks;
+  const int ld_row = tid / kRowChunks, ld_col = tid % kRowChunks;
+  const uint32_t k_rel = (uint32_t)(ld_row * k_tok_b) + ld_col * 16;
+  const uint32_t v_rel = (uint32_t)(ld_row * v_tok_b) + ld_col * 16;
   auto fetch = [&](int tile) {
+    const int64_t t0 = (int64_t)tile * kPfKeys;
+    if (t0 + kPfKeys - 1 <= last_key) {             // a whole tile: one base, constant offsets
+      const char *kt0 = kbase + t0 * k_tok_b, *vt0 = vbase + t0 * v_tok_b;
 #pragma unroll
-    for (int u = 0; u < kLoads; ++u) {
-      const int chunk = tid + u * kPfThreads;
-      const int row = chunk / kRowChunks, col = chunk % kRowChunks;
-      int64_t tok = (int64_t)tile * kPfKeys + row;
-      if (tok > last_key) tok = last_key;           // in bounds; such keys are masked
-      kst[u] = load16(kbase + tok * k_tok_b + col * 16);
-      vst[u] = load16(vbase + tok * v_tok_b + col * 16);
+      for (int u = 0; u < kLoads; ++u) {
+        kst[u] = load16(kt0 + (k_rel + (uint32_t)(u * kRowsPerLoad * k_tok_b)));
+        vst[u] = load16(vt0 + (v_rel + (uint32_t)(u * kRowsPerLoad * v_tok_b)));
+      }
+    } else {                                        // the ragged last tile: rows clamped into range
+#pragma unroll
+      for (int u = 0; u < kLoads; ++u) {
+        int64_t tok = t0 + ld_row + u * kRowsPerLoad;
+        if (tok > last_key) tok = last_key;         // in bounds; such keys are masked
+        kst[u] = load16(kbase + tok * k_tok_b + ld_col * 16);
+        vst[u] = load16(vbase + tok * v_tok_b + ld_col * 16);
+      }
     }
   };
   auto stage = [&](int buf) {
@@ -254,6 +268,10 @@ prefill_attention_kernel(const PrefillArgs a) {
   };
 
   fetch(0);
+  // The query rows have arrived before the loop starts (they were requested ahead of
+  // tile 0): inside the loop nothing then waits for a load except the tile's own.
+#pragma unroll
+  for (int s = 0; s < kQSteps; ++s) asm volatile("" : "+v"(qf[s]));
   stage(0);
   __syncthreads();
   for (int tile = 0; tile < n_tiles; ++tile) {
@@ -341,6 +359,8 @@ extern "C" int da_prefill_attention(const void *q, int64_t q_tok_stride, int64_t
                  o_tok_stride % 8 == 0 && o_head_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
                  (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 && (uintptr_t)out % 16 == 0,
              "da_prefill_attention: rows must be 16-byte aligned");
+  if (k_tok_stride < 0 || v_tok_stride < 0 || k_tok_stride > (1 << 23) || v_tok_stride > (1 << 23))
+    return fail(DA_ENOTSUP, "da_prefill_attention: key/value token strides of 0..2^23 elements");
   PrefillArgs a = {};
   a.q = (const char *)q;
   a.k = (const char *)k;
