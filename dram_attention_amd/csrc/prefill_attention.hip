@@ -24,9 +24,9 @@
 // Q^T stays in registers for the whole pass; K rows are the A operand of the
 // first product straight from the LDS tile (one 16-byte read per MFMA).
 //
-// The next tile's K/V rows travel global memory -> registers while the current
-// tile is computed, and registers -> the other LDS buffer afterwards: one
-// barrier per tile.  Softmax state per query row: a running reference m that
+// The next tile's K/V rows travel from global memory straight into the other LDS
+// buffer (loads that write LDS, no registers in between) while the current tile is
+// computed: one barrier per tile.  Softmax state per query row: a running reference m that
 // is only raised when a score clears it by kRescaleSlack (as in the decode
 // kernels), per-lane partial sums, everything in the log2 domain.
 // Workgroups are numbered kv head by kv head, the longest rows of a head first.
@@ -81,20 +81,32 @@ constexpr int kPfThreads = 256;
 constexpr int kPfWaves = 4;
 constexpr int kPfKeys = 64;  // keys per tile
 
+// LDS layout of a tile.  K and V rows arrive by loads that write LDS directly
+// (global_load_lds_dwordx4: no staging registers, no LDS store instructions): a wave
+// instruction deposits its 64 lanes' 16-byte chunks at 64 consecutive places, one block
+// of 1024 bytes = kRows rows.  Which chunk a lane fetches is free, so the chunks of a
+// block are placed with their column index XORed by a function of the row: the 16
+// lanes that read one column of 16 rows (K rows as MFMA operands), and the 8 rows x 64
+// bytes of a transposing read of V, then fall on distinct banks; 16 bytes of padding
+// per block shift consecutive blocks by one bank group.
 template <int kD>
 struct PrefillShared {
-  // K rows are read 16 bytes per lane by 32 lanes at one column: a row stride of
-  // 16 bytes mod 256 spreads them over the banks.  V rows are read by the
-  // transposing load, 8 bytes per lane, four rows by 64 bytes at a time: 64 bytes
-  // mod 256.
-  static constexpr int kKRow = kD * 2 + 16;
-  static constexpr int kVRow = kD * 2 + 64;
-  static constexpr int kKBytes = kPfKeys * kKRow;
-  static constexpr int kVBytes = kPfKeys * kVRow;
-  static constexpr int kBufBytes = kKBytes + kVBytes;
-  static constexpr int kOutRow = kD * 2 + 16;                     // epilogue staging
+  static constexpr int kRowBytes = kD * 2;
+  static constexpr int kRows = 1024 / kRowBytes;          // rows per block: 4 (D 128) or 8 (D 64)
+  static constexpr int kChunks = kRowBytes / 16;          // 16-byte chunks per row
+  static constexpr int kBlock = 1024 + 16;                // bytes from block to block
+  static constexpr int kBlocks = kPfKeys / kRows;         // blocks per tile (K, and V)
+  static constexpr int kKBytes = kBlocks * kBlock;
+  static constexpr int kBufBytes = 2 * kKBytes;           // K tile, then V tile
+  static constexpr int kOutRow = kD * 2 + 16;             // epilogue staging
   static constexpr int kOutBytes = kPfWaves * 32 * kOutRow;
   static constexpr int kBytes = 2 * kBufBytes > kOutBytes ? 2 * kBufBytes : kOutBytes;
+  // column swizzle of row rr of a block (a multiple of the chunk index's high bits)
+  static __host__ __device__ constexpr int swizzle(int rr) { return kD == 128 ? 4 * rr : 2 * (rr >> 1); }
+  // byte offset of chunk cc of row r of a tile
+  static __device__ __forceinline__ int at(int r, int cc) {
+    return (r / kRows) * kBlock + (r % kRows) * kRowBytes + ((cc ^ swizzle(r % kRows)) * 16);
+  }
 };
 
 template <typename T, int kD, int kHeads>
@@ -147,43 +159,63 @@ prefill_attention_kernel(const PrefillArgs a) {
   const char *vbase = a.v + (int64_t)hk * a.v_head_stride * T::kBytes;
   const int64_t k_tok_b = a.k_tok_stride * T::kBytes, v_tok_b = a.v_tok_stride * T::kBytes;
 
-  // This thread's 16-byte chunks of a tile: chunk tid + 256*u = row tid/kRowChunks + u*(256/kRowChunks),
-  // column tid%kRowChunks.  Offsets inside a tile fit 32 bits (checked by the launcher).
-  u32x4 kst[kLoads], vst[kLoads];
-  constexpr int kRowsPerLoad = kPfThreads / kRowChunks;
-  const int ld_row = tid / kRowChunks, ld_col = tid % kRowChunks;
+  // Tile loads.  Wave w brings blocks w, w + 4, ... of K and of V; lane L of the wave
+  // owns place L of a block, i.e. row L / kChunks and the chunk whose swizzled column is
+  // L % kChunks.  Offsets inside a tile fit 32 bits (checked by the launcher).
+  constexpr int kBlocksPerWave = Sh::kBlocks / kPfWaves;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int ld_row = lane / Sh::kChunks;
+  const int ld_col = (lane % Sh::kChunks) ^ Sh::swizzle(ld_row);
   const uint32_t k_rel = (uint32_t)(ld_row * k_tok_b) + ld_col * 16;
   const uint32_t v_rel = (uint32_t)(ld_row * v_tok_b) + ld_col * 16;
-  auto fetch = [&](int tile) {
+  typedef __attribute__((address_space(1))) const void *GlobalPtr;
+  typedef __attribute__((address_space(3))) void *LdsPtr;
+  auto fetch = [&](int tile, int buf) {
     const int64_t t0 = (int64_t)tile * kPfKeys;
+    char *kt = smem + buf * Sh::kBufBytes;
     if (t0 + kPfKeys - 1 <= last_key) {             // a whole tile: one base, constant offsets
       const char *kt0 = kbase + t0 * k_tok_b, *vt0 = vbase + t0 * v_tok_b;
 #pragma unroll
-      for (int u = 0; u < kLoads; ++u) {
-        kst[u] = load16(kt0 + (k_rel + (uint32_t)(u * kRowsPerLoad * k_tok_b)));
-        vst[u] = load16(vt0 + (v_rel + (uint32_t)(u * kRowsPerLoad * v_tok_b)));
+      for (int u = 0; u < kBlocksPerWave; ++u) {
+        const int blk = wave_u + u * kPfWaves;
+        __builtin_amdgcn_global_load_lds(
+            (GlobalPtr)(kt0 + (int64_t)blk * Sh::kRows * k_tok_b + k_rel),
+            (LdsPtr)(kt + blk * Sh::kBlock), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(
+            (GlobalPtr)(vt0 + (int64_t)blk * Sh::kRows * v_tok_b + v_rel),
+            (LdsPtr)(kt + Sh::kKBytes + blk * Sh::kBlock), 16, 0, 0);
       }
     } else {                                        // the ragged last tile: rows clamped into range
 #pragma unroll
-      for (int u = 0; u < kLoads; ++u) {
-        int64_t tok = t0 + ld_row + u * kRowsPerLoad;
+      for (int u = 0; u < kBlocksPerWave; ++u) {
+        const int blk = wave_u + u * kPfWaves;
+        int64_t tok = t0 + blk * Sh::kRows + ld_row;
         if (tok > last_key) tok = last_key;         // in bounds; such keys are masked
-        kst[u] = load16(kbase + tok * k_tok_b + ld_col * 16);
-        vst[u] = load16(vbase + tok * v_tok_b + ld_col * 16);
+        __builtin_amdgcn_global_load_lds((GlobalPtr)(kbase + tok * k_tok_b + ld_col * 16),
+                                         (LdsPtr)(kt + blk * Sh::kBlock), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((GlobalPtr)(vbase + tok * v_tok_b + ld_col * 16),
+                                         (LdsPtr)(kt + Sh::kKBytes + blk * Sh::kBlock), 16, 0, 0);
       }
     }
   };
-  auto stage = [&](int buf) {
-    char *kt = smem + buf * Sh::kBufBytes;
-    char *vt = kt + Sh::kKBytes;
+
+  // LDS addresses of this lane's operands inside a tile.  K, as the A operand of S^T:
+  // row c of a half, chunk 2s + g.  V, for the transposing load: lane i of a 16-lane
+  // group addresses key t0 + i/4, channels c0 + 4*(i%4) .. +3 and receives channel
+  // c0 + i of keys t0..t0+3; t0 = 4g (+8, +16 per group of keys), c0 = 32b + 16*((lane/16)%2).
+  int k_at[kQSteps], v_at[kCBlocks];
 #pragma unroll
-    for (int u = 0; u < kLoads; ++u) {
-      const int chunk = tid + u * kPfThreads;
-      const int row = chunk / kRowChunks, col = chunk % kRowChunks;
-      *(u32x4 *)(kt + row * Sh::kKRow + col * 16) = kst[u];
-      *(u32x4 *)(vt + row * Sh::kVRow + col * 16) = vst[u];
-    }
-  };
+  for (int s2 = 0; s2 < kQSteps; ++s2) k_at[s2] = Sh::at(c, 2 * s2 + g);
+  {
+    const int i16 = lane & 15;
+#pragma unroll
+    for (int b = 0; b < kCBlocks; ++b)
+      v_at[b] = Sh::kKBytes + Sh::at(4 * g + (i16 >> 2), 4 * b + 2 * ((lane >> 4) & 1) + ((i16 & 3) >> 1)) +
+                (i16 & 1) * 8;
+  }
+  constexpr int kHalfStep = (32 / Sh::kRows) * Sh::kBlock;   // 32 rows further down a tile
+  constexpr int kKeys16 = (16 / Sh::kRows) * Sh::kBlock;     // 16 rows
+  constexpr int kKeys8 = (8 / Sh::kRows) * Sh::kBlock;       // 8 rows
 
   float m = kMinusHuge, l = 0.f;
   pf_f32x16 acc[kCBlocks];
@@ -196,16 +228,19 @@ prefill_attention_kernel(const PrefillArgs a) {
   auto compute = [&](int tile, int buf, auto mask_tag) {
     constexpr bool kMask = decltype(mask_tag)::value;
     const char *kt = smem + buf * Sh::kBufBytes;
-    const char *vt = kt + Sh::kKBytes;
     pf_f32x16 st[2];
+    // (raised priority while a wave issues MFMAs: they go ahead of the vector work of the
+    // other wave on this SIMD, which fills the gaps; +2.5 %)
+    __builtin_amdgcn_s_setprio(3);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) st[half][i] = 0.f;
-      const char *kr = kt + (half * 32 + c) * Sh::kKRow + g * 16;
 #pragma unroll
-      for (int s = 0; s < kQSteps; ++s) st[half] = Ops::mma(*(const u32x4 *)(kr + s * 32), qf[s], st[half]);
+      for (int s = 0; s < kQSteps; ++s)
+        st[half] = Ops::mma(*(const u32x4 *)(kt + k_at[s] + half * kHalfStep), qf[s], st[half]);
     }
+    __builtin_amdgcn_s_setprio(0);
     // register 4j + i of half `half`: key tile*64 + half*32 + 8j + 4g + i
     float smax = -INFINITY;
     if constexpr (kMask) {
@@ -248,43 +283,39 @@ prefill_attention_kernel(const PrefillArgs a) {
         pt[half * 2 + jj] = u32x4{Ops::pack(p[8 * jj], p[8 * jj + 1]), Ops::pack(p[8 * jj + 2], p[8 * jj + 3]),
                                   Ops::pack(p[8 * jj + 4], p[8 * jj + 5]), Ops::pack(p[8 * jj + 6], p[8 * jj + 7])};
     }
-    // V^T operands by the transposing load: lane i of a 16-lane group addresses key
-    // t0 + i/4, channels c0 + 4*(i%4) .. +3 and receives channel c0 + i of keys t0..t0+3
-    const int i16 = lane & 15;
-    const char *vr = vt + (4 * g + (i16 >> 2)) * Sh::kVRow + (((lane >> 4) & 1) * 16 + (i16 & 3) * 4) * 2;
+    __builtin_amdgcn_s_setprio(3);
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {   // 16 keys each
 #pragma unroll
       for (int b = 0; b < kCBlocks; ++b) {
-        const char *p0 = vr + (kk * 16) * Sh::kVRow + b * 64;
+        const char *p0 = kt + v_at[b] + kk * kKeys16;
         const pf_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (pf_i16x4 __attribute__((address_space(3))) *)(p0));
         const pf_i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (pf_i16x4 __attribute__((address_space(3))) *)(p0 + 8 * Sh::kVRow));
+            (pf_i16x4 __attribute__((address_space(3))) *)(p0 + kKeys8));
         const u32x4 va = __builtin_bit_cast(u32x4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         acc[b] = Ops::mma(va, pt[kk], acc[b]);
       }
     }
+    __builtin_amdgcn_s_setprio(0);
   };
 
-  fetch(0);
+  fetch(0, 0);
   // The query rows have arrived before the loop starts (they were requested ahead of
   // tile 0): inside the loop nothing then waits for a load except the tile's own.
 #pragma unroll
   for (int s = 0; s < kQSteps; ++s) asm volatile("" : "+v"(qf[s]));
-  stage(0);
-  __syncthreads();
+  __syncthreads();                                  // (waits for this wave's tile loads first)
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int buf = tile & 1;
-    const bool more = tile + 1 < n_tiles;
-    if (more) fetch(tile + 1);
+    // the other buffer was last read before the barrier that ended the previous round
+    if (tile + 1 < n_tiles) fetch(tile + 1, buf ^ 1);
     const int64_t t0 = (int64_t)tile * kPfKeys;
     if (t0 <= wave_last_key) {                     // else: every key of the tile is masked for this wave
       if (t0 + kPfKeys - 1 > row0) compute(tile, buf, std::true_type{});
       else compute(tile, buf, std::false_type{});
     }
-    if (more) stage(buf ^ 1);
-    __syncthreads();
+    __syncthreads();                                // tile + 1 has landed, and everyone is done with `buf`
   }
 
   // ---- epilogue: normalise, transpose through LDS, store rows of 16-byte lanes
