@@ -230,7 +230,7 @@ prefill_attention_kernel(const PrefillArgs a) {
     const char *kt = smem + buf * Sh::kBufBytes;
     pf_f32x16 st[2];
     // (raised priority while a wave issues MFMAs: they go ahead of the vector work of the
-    // other wave on this SIMD, which fills the gaps; +2.5 %)
+    // other wave on this SIMD, which fills the gaps; worth 0-2 % from run to run)
     __builtin_amdgcn_s_setprio(3);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
