@@ -91,6 +91,32 @@ def test_prefill_attention_takes_strided_views_and_peaked_scores():
     assert same(out[0, 0].view(Hkv, Hq // Hkv, D), xv[0, 0][:, None].expand(-1, Hq // Hkv, -1))
 
 
+def test_prefill_attention_at_the_headline_prompt_length_on_sampled_rows():
+    """configs[2]'s prompt (135 152 tokens, 32 q / 8 kv heads, D 128, bf16) through the
+    kernel once; rows sampled from the first, a middle and the last blocks, and around
+    tile boundaries, are held against a dense fp32 causal softmax over all their keys."""
+    from dram_attention_amd.dram_attention import prefill_attention
+
+    S, Hq, Hkv, D = 131072 + 4096 - 16, 32, 8, 128
+    rep = Hq // Hkv
+    xq, xk, xv = draw(S, Hq, Hkv, D, torch.bfloat16, 5)
+    lse = torch.empty(Hq, S, dtype=torch.float32, device=DEV)
+    out = prefill_attention(xq, xk, xv, lse=lse)
+    rows = torch.tensor(sorted(set(
+        list(range(0, 70)) + list(range(65500, 65570)) + [4095, 4096, 4097, 100000, 100063, 100064, 131071, 131072]
+        + list(range(S - 40, S)))), device=DEV)
+    scale = 1.0 / math.sqrt(D)
+    for h in range(Hkv):
+        q = xq[0, rows, h * rep:(h + 1) * rep].float().transpose(0, 1)       # (rep, R, D)
+        s_ = torch.matmul(q, xk[0, :, h].float().t()) * scale                 # (rep, R, S)
+        keys = torch.arange(S, device=DEV)
+        s_.masked_fill_(keys[None, None, :] > rows[None, :, None], float("-inf"))
+        want = torch.matmul(torch.softmax(s_, dim=-1), xv[0, :, h].float()).transpose(0, 1)   # (R, rep, D)
+        assert close(out[0, rows, h * rep:(h + 1) * rep].float(), want, ATOL, RTOL)
+        assert close(lse[h * rep:(h + 1) * rep][:, rows], torch.logsumexp(s_, dim=-1), 1e-3, 1e-4)
+    assert torch.isfinite(out.float()).all()
+
+
 def test_prefill_attention_rejects_what_the_kernel_does_not_cover():
     from dram_attention_amd.dram_attention import (causal_prefill_attention, prefill_attention,
                                                    prefill_attention_supported)
