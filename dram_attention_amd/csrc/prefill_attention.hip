@@ -29,7 +29,8 @@
 // computed: one barrier per tile.  Softmax state per query row: a running reference m that
 // is only raised when a score clears it by kRescaleSlack (as in the decode
 // kernels), per-lane partial sums, everything in the log2 domain.
-// Workgroups are numbered kv head by kv head, the longest rows of a head first.
+// Workgroups take the longest rows first; which kv head a workgroup works on follows the
+// die it runs on where the heads deal out evenly over the dies (see the kernel).
 #include <type_traits>
 
 #include "attention_core.hpp"
@@ -74,12 +75,14 @@ struct PrefillArgs {
   int rep;          // query heads per kv head
   int n_groups;     // workgroups that share a kv head's rows: rep / kHeads
   int64_t n_row_blocks;
+  int heads_per_xcd;  // kv heads per die when they deal out evenly, else 0
   float scale_log2;
 };
 
 constexpr int kPfThreads = 256;
 constexpr int kPfWaves = 4;
 constexpr int kPfKeys = 64;  // keys per tile
+constexpr int kXcds = 8;     // dies (XCDs) of the part; consecutive workgroup ids go to consecutive dies
 
 // LDS layout of a tile.  K and V rows arrive by loads that write LDS directly
 // (global_load_lds_dwordx4: no staging registers, no LDS store instructions): a wave
@@ -128,10 +131,22 @@ prefill_attention_kernel(const PrefillArgs a) {
   const int g = lane >> 5;
   const int c = lane & 31;
 
-  // workgroup -> (kv head, row block, head group): kv head slowest, long rows first
+  // workgroup -> (kv head, row block, head group), long rows first.  Workgroups are dealt
+  // to the chip's kXcds dies in turn and every die has a cache of its own: with a multiple
+  // of kXcds kv heads, workgroup b works on a head that is b's die's alone (b % kXcds,
+  // + kXcds, ...), so that a die's cache holds the keys and values of one head at a time
+  // and no two dies fetch the same rows.  Otherwise: kv head by kv head.
   const int64_t per_head = a.n_row_blocks * a.n_groups;
-  const int hk = (int)(blockIdx.x / per_head);
-  const int64_t rem = blockIdx.x % per_head;
+  int hk;
+  int64_t rem;
+  if (a.heads_per_xcd > 0) {
+    const int64_t j = blockIdx.x / kXcds;               // this die's j-th workgroup
+    hk = (int)(blockIdx.x % kXcds) + kXcds * (int)(j / per_head);
+    rem = j % per_head;
+  } else {
+    hk = (int)(blockIdx.x / per_head);
+    rem = blockIdx.x % per_head;
+  }
   const int64_t rb = a.n_row_blocks - 1 - rem / a.n_groups;
   const int hg = (int)(rem % a.n_groups);
   const int hq = hk * a.rep + hg * kHeads + wave % kHeads;
@@ -351,6 +366,7 @@ static int launch_prefill(PrefillArgs a, int n_kv_heads, hipStream_t s) {
   const int block_rows = 32 * (kPfWaves / heads);
   a.n_groups = a.rep / heads;
   a.n_row_blocks = ceil_div(a.seq_len, block_rows);
+  a.heads_per_xcd = n_kv_heads % kXcds == 0 ? n_kv_heads / kXcds : 0;
   const int64_t blocks = a.n_row_blocks * a.n_groups * n_kv_heads;
   if (blocks > 0x7fffffff) return fail(DA_ENOTSUP, "da_prefill_attention: %lld workgroups", (long long)blocks);
   const dim3 grid((unsigned)blocks);
