@@ -7,9 +7,11 @@
 // per query head); K and V are re-read once per block of query rows, from the
 // memory-side cache while one kv head's 2*S*D*e bytes fit it.
 //
-// Work split: a 256-thread workgroup owns kHeads query heads of one kv head
-// (the GQA group, or a part of it) times 128/kHeads consecutive query rows;
-// each of its four waves owns 32 query rows of one head.  All waves walk the
+// Work split: a 512-thread workgroup, one per CU, owns kHeads query heads of one kv
+// head (the GQA group, or a part of it) times 256/kHeads consecutive query rows;
+// each of its eight waves owns 32 query rows of one head (two waves per SIMD: the
+// registers of a wave allow no more, and with eight waves on one tile instead of two
+// workgroups of four on two the CU loads half as many tile rows).  All waves walk the
 // same keys, so one tile of K and V in LDS serves the whole group.  Per tile
 // of 64 keys a wave computes, with 32x32x16 MFMAs,
 //   S^T (keys x rows)  = K (keys x D) * Q^T (D x rows)        D/16 per 32 keys
@@ -79,8 +81,8 @@ struct PrefillArgs {
   float scale_log2;
 };
 
-constexpr int kPfThreads = 256;
-constexpr int kPfWaves = 4;
+constexpr int kPfThreads = 512;
+constexpr int kPfWaves = 8;
 constexpr int kPfKeys = 64;  // keys per tile
 constexpr int kXcds = 8;     // dies (XCDs) of the part; consecutive workgroup ids go to consecutive dies
 
@@ -113,7 +115,7 @@ struct PrefillShared {
 };
 
 template <typename T, int kD, int kHeads>
-__global__ void __launch_bounds__(kPfThreads, 2)
+__global__ void __launch_bounds__(kPfThreads, 1)
 prefill_attention_kernel(const PrefillArgs a) {
   using Ops = PrefillOps<T>;
   using Sh = PrefillShared<kD>;
