@@ -200,8 +200,10 @@ def causal_prefill_attention(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tenso
       "native"  the library's kernel (16-bit types, head_dim 64 or 128; raises otherwise)
       "sdpa"    torch's fused scaled_dot_product_attention (raises if no fused kernel
                 takes the shape)
-      "blocked" torch's attention over blocks of 1024 query rows with an explicit mask,
-                so that no S x S score matrix is ever materialised (any type, CPU too)
+      "blocked" torch's attention over blocks of query rows with an explicit mask, the
+                block sized so that the scores torch may materialise for it (Hq x rows x S
+                fp32) stay within 1 GiB: at most 1024 rows, 64 at 128K tokens and 32
+                heads (any type, CPU too)
       "auto"    native where it applies, else sdpa, else blocked."""
     if backend not in ("auto", "native", "sdpa", "blocked"):
         raise RuntimeError(f"Unsupported prefill backend: {backend}")
@@ -224,7 +226,7 @@ def causal_prefill_attention(xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tenso
             if backend == "sdpa":
                 raise
     out = torch.empty_like(xq)
-    block = 1024
+    block = max(16, min(1024, (1 << 28) // max(1, Hq * S)))
     for s0 in range(0, S, block):
         s1 = min(S, s0 + block)
         # rows s0..s1 see keys 0..s1; row i of the block may look at key j <= s0 + i

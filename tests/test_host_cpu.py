@@ -258,3 +258,23 @@ def test_bench_roofline_traffic_constant_matches_the_committed_counter_summary()
     assert parsed is not None and parsed == bench.ROOFLINE_TRAFFIC_BYTES["128k"]
     assert 151.26e6 <= parsed < 1.1 * 151.26e6      # at least the algorithmic bytes, little more
     assert bench.roofline_traffic_from_profile(os.path.join(ROOT, "profiles", "no_such_file.md")) is None
+
+
+def test_blocked_prefill_fallback_on_cpu_matches_dense_causal_softmax():
+    """The torch fallback of the prefill stage (what fp32 or an odd head_dim takes) against
+    a dense causal softmax, with a block size small enough to cross several blocks."""
+    import math
+
+    import torch
+
+    from dram_attention_amd.dram_attention import causal_prefill_attention
+
+    torch.manual_seed(0)
+    S, Hq, Hkv, D = 2500, 4, 2, 16
+    q, k, v = torch.randn(1, S, Hq, D), torch.randn(1, S, Hkv, D), torch.randn(1, S, Hkv, D)
+    got = causal_prefill_attention(q, k, v, "blocked")
+    kk, vv = k.repeat_interleave(Hq // Hkv, 2), v.repeat_interleave(Hq // Hkv, 2)
+    sc = torch.einsum("bqhd,bkhd->bhqk", q, kk) / math.sqrt(D)
+    sc = sc.masked_fill(~torch.ones(S, S, dtype=torch.bool).tril(), float("-inf"))
+    want = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(sc, -1), vv)
+    assert torch.allclose(got, want, atol=1e-5, rtol=1e-5)
