@@ -4,8 +4,8 @@
 // of the reference.
 //
 // Bound: MFMA.  4*S*S*D*Hq/2 flops (the causal half of two S x S x D products
-// per query head); K and V are re-read once per block of query rows, from the
-// memory-side cache while one kv head's 2*S*D*e bytes fit it.
+// per query head); K and V are re-read once per block of query rows, nearly always
+// from the L2 of the die the workgroup runs on (its neighbours there walk the same keys).
 //
 // Work split: a 512-thread workgroup, one per CU, owns kHeads query heads of one kv
 // head (the GQA group, or a part of it) times 256/kHeads consecutive query rows;
