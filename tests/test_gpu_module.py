@@ -229,6 +229,56 @@ def test_prefill_call_then_generate_matches_oracle():
         assert close(got.cpu().float(), want.float(), 2e-2, 1e-2), f"step {t}"
 
 
+def test_prefill_call_at_the_headline_size_builds_the_same_layer_as_init_cache():
+    """configs[2] as a model would run it: forward(stage="prefill") over the whole
+    135 152-token prompt (the library's causal kernel, summaries, page store, slots), then
+    generate calls.  The state the call leaves is bit-equal to what init_cache builds from
+    the same K/V, the decode steps that follow are bit-equal too, and the prefill output
+    is held against a dense fp32 causal softmax on sampled rows."""
+    from dram_attention_amd import DRAMAttention
+
+    w = WORKLOADS["128k"]
+    prompt = make_prompt(w, 31)
+    S = w.prompt_tokens
+    g = torch.Generator(device=DEV).manual_seed(32)
+    xq0 = torch.randn(1, S, w.n_q_heads, w.head_dim, device=DEV, generator=g).to(w.dtype)
+    k, v = prompt.k.to(DEV), prompt.v.to(DEV)
+
+    def layer():
+        return DRAMAttention(8, w.lru_tokens, w.local_cache, w.page_size, w.top_k_tokens,
+                             w.n_kv_heads, w.head_dim, device=DEV, dtype=w.dtype)
+
+    m, r = layer(), layer()
+    out0 = m(xq0, k, v, start_pos=0, stage="prefill")
+    r.init_cache(k, v)
+    assert out0.shape == xq0.shape and m.dram_kv_cache_size == r.dram_kv_cache_size
+    for name in ("dram_kv_cache", "hbm_kv_cache", "page_access_time", "dram_page_to_hbm_page_mapping",
+                 "hbm_page_to_dram_page_mapping"):
+        assert same(getattr(m.lru_cache, name), getattr(r.lru_cache, name)), name
+    assert same(m.cache_k, r.cache_k) and same(m.cache_v, r.cache_v)
+    assert same(m.lru_cache.top_k_selector.chunk_min_max, r.lru_cache.top_k_selector.chunk_min_max)
+
+    # the prefill output on sampled rows of every head
+    rep = w.n_q_heads // w.n_kv_heads
+    rows = torch.tensor(sorted(set(list(range(0, 40)) + [4095, 4096, 65535, 65536, 100000] + list(range(S - 40, S)))),
+                        device=DEV)
+    keys = torch.arange(S, device=DEV)
+    for h in range(w.n_kv_heads):
+        q = xq0[0, rows, h * rep:(h + 1) * rep].float().transpose(0, 1)
+        sc = torch.matmul(q, k[0, :, h].float().t()) / math.sqrt(w.head_dim)
+        sc.masked_fill_(keys[None, None, :] > rows[None, :, None], float("-inf"))
+        want = torch.matmul(torch.softmax(sc, dim=-1), v[0, :, h].float()).transpose(0, 1)
+        assert close(out0[0, rows, h * rep:(h + 1) * rep].float(), want, 2e-2, 1e-2)
+
+    inputs = DecodeInputs(w, prompt.q0, 31)
+    for t in range(3):
+        xq, xk, xv = (x.to(DEV) for x in inputs.next())
+        got = m(xq, xk, xv, start_pos=S + t, stage="generate")
+        ref = r(xq, xk, xv, start_pos=S + t, stage="generate")
+        assert same(got, ref), f"step {t}"
+        assert same(m.lru_cache._topk_idx, r.lru_cache._topk_idx)
+
+
 # ------------------------------------------------------------ whole decode runs vs the oracle
 def run_parity(w, seed, steps, atol, rtol, device_pos=False):
     """Drives the module and the oracle with the same inputs.  Selection and LRU
