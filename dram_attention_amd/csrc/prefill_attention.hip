@@ -126,7 +126,6 @@ prefill_attention_kernel(const PrefillArgs a) {
   constexpr int kQSteps = kD / 16;                    // MFMAs of S^T per 32 keys
   constexpr int kCBlocks = kD / 32;                   // 32-channel blocks of O^T
   constexpr int kRowChunks = kD / 8;                  // 16-byte chunks per K/V row
-  constexpr int kLoads = kPfKeys * kRowChunks / kPfThreads;  // 16-byte loads per thread and tile (K, and V)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
